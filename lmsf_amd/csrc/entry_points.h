@@ -37,16 +37,18 @@ int lmsf_latent_cache_write(const void* x, int dtype, long x_stride, const float
     int Q, hipStream_t stream);
 int lmsf_head_linear(const void* x, int dtype, long x_stride, int x_head, const void* W, void* y, long y_stride,
     int y_head, const void* gate, long gate_stride, int n_tokens, int H, int O, int K, const int* positions,
-    const float* table, int rot, int max_pos, int x_at, int y_at, int dr, hipStream_t stream);
+    const float* table, int rot, int max_pos, int x_at, int y_at, int dr, int gate_wide, hipStream_t stream);
 int lmsf_rope_tail(const void* x, int dtype, long x_stride, int x_head, int x_at, void* y, long y_stride, int y_head,
     int y_at, const int* positions, const float* table, int rot, int max_pos, int n_tokens, int H, int dr,
     hipStream_t stream);
 
 // moe.hip
 int lmsf_table_moe(const void* h, int dtype, long h_stride, const void* Wgu, const void* Wd, const int* ids,
-    const int* table, int vocab, int top, int E, float weight, const void* base, long base_stride, void* act,
-    void* out, long out_stride, int n_tokens, int F, int W, int* scratch_ints, float* scratch_rows,
-    hipStream_t stream);
+    const int* table, int vocab, int top, int E, float weight, const void* base, long base_stride,
+    const float* pair_scale, const float* base_scale, void* act, void* out, long out_stride, int n_tokens, int F,
+    int W, int* scratch_ints, float* scratch_rows, hipStream_t stream);
+int lmsf_moe_route(const float* z, long z_stride, int n_tokens, int E, int top, int renorm, int extra, int* choice,
+    float* weight, float* gate, hipStream_t stream);
 long lmsf_table_moe_scratch_ints(int n_tokens, int top, int E);
 int lmsf_table_moe_grouped(int dtype, int n_tokens, int top, int E, int F, int W, long h_stride);
 
@@ -194,6 +196,27 @@ int lmsf_sample(const float* logits, long ld, int R, int V, const float* tempera
 int lmsf_apply_penalties(float* logits, long ld, int R, int V, const int* tokens, const int* offsets, const int*
     prompt_lens, int* counts, const float* presence, const float* frequency, const float* repetition, hipStream_t
     stream);
+
+// retention.hip
+long lmsf_retention_state_floats(int H, int d, int dv);
+int lmsf_retention_chunk_tokens(int d);
+long lmsf_retention_chunk_entry_floats(int H, int d, int dv);
+int lmsf_retention_chunked(const void* q, const void* k, const void* v, int dtype, long qkv_stride,
+    const int* positions, const float* table, int rot, int max_pos, const float* decay, const void* og,
+    long og_stride, float* state, long state_stride, const int* seg_starts, const int* state_slots, void* out,
+    long out_stride, float* o_raw, int n_tokens, int n_segments, int H, int d, int dv, float qscale, float eps,
+    const int* chunk_base, int max_chunks, long n_entries, float* entries, hipStream_t stream);
+int lmsf_retention_tokens(const void* q, const void* k, const void* v, int dtype, long qkv_stride,
+    const int* positions, const float* table, int rot, int max_pos, const float* decay, const void* og,
+    long og_stride, float* state, long state_stride, const int* seg_starts, const int* state_slots, void* out,
+    long out_stride, float* o_raw, int n_tokens, int n_segments, int H, int d, int dv, float qscale, float eps,
+    hipStream_t stream);
+
+// layer_scale.hip
+int lmsf_scale_add_norm(const void* a, long a_stride, const float* sa, const void* b, long b_stride, const float* sb,
+    int dtype, float* stream, const void* wn, int wn_dtype, void* out, int n_rows, int W, float eps,
+    hipStream_t stream_);
+int lmsf_logit_cap(float* logits, long stride, int R, int V, float scale, float cap, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -10,7 +10,8 @@
 //
 //   lmsf_latent_cache_write   c = rms_norm(x[:R]) * w, r = rotate(x[R:R+dr]) -> pages at the token's slot; from the
 //                             same launch the norm of the query's latent, which lies in the same row of the product
-//   lmsf_head_linear          y[n, h, :] = W_h x[n, h, :K] (* sigmoid(gate[n, h])), W [H, O, K]: per-head products
+//   lmsf_head_linear          y[n, h, :] = W_h x[n, h, :K] (* sigmoid(gate[n, h]), or with ``gate_wide`` entry by
+//                             entry * sigmoid(gate[n, h * O + o])), W [H, O, K]: per-head products
 //                             (32 tokens and more in bfloat16: on the matrix cores)
 //   lmsf_rope_tail            rotates one part of every head of q into another buffer and zeroes its padding
 //
@@ -118,7 +119,7 @@ extern "C" int lmsf_latent_cache_write(const void* x, int dtype, long x_stride, 
 template <typename T>
 __global__ __launch_bounds__(LAT_THREADS) void head_linear_kernel(
     const T* __restrict__ x, long x_stride, int x_head, const T* __restrict__ W, T* __restrict__ y, long y_stride,
-    int y_head, const T* __restrict__ gate, long gate_stride, int n_tokens, int O, int K, int vec) {
+    int y_head, const T* __restrict__ gate, long gate_stride, int n_tokens, int O, int K, int vec, int gate_wide) {
   extern __shared__ float sx[];   // [HL_TOKENS, K]
   const int h = blockIdx.y, n0 = blockIdx.x * HL_TOKENS;
   const int nt = min(HL_TOKENS, n_tokens - n0);
@@ -131,7 +132,7 @@ __global__ __launch_bounds__(LAT_THREADS) void head_linear_kernel(
 #pragma unroll
   for (int t = 0; t < HL_TOKENS; ++t) {
     g[t] = 1.f;
-    if (gate && t < nt) g[t] = 1.f / (1.f + expf(-to_f32<T>(gate[(long)(n0 + t) * gate_stride + h])));
+    if (gate && !gate_wide && t < nt) g[t] = 1.f / (1.f + expf(-to_f32<T>(gate[(long)(n0 + t) * gate_stride + h])));
   }
   const T* Wh = W + (long)h * O * K;
   constexpr int V = Vec16<T>::N;
@@ -161,7 +162,11 @@ __global__ __launch_bounds__(LAT_THREADS) void head_linear_kernel(
     }
 #pragma unroll
     for (int t = 0; t < HL_TOKENS; ++t)
-      if (t < nt) y[(long)(n0 + t) * y_stride + (long)h * y_head + o] = from_f32<T>(acc[t] * g[t]);
+      if (t < nt) {
+        const float gg = gate && gate_wide
+            ? 1.f / (1.f + expf(-to_f32<T>(gate[(long)(n0 + t) * gate_stride + (long)h * O + o]))) : g[t];
+        y[(long)(n0 + t) * y_stride + (long)h * y_head + o] = from_f32<T>(acc[t] * gg);
+      }
   }
 }
 
@@ -196,7 +201,7 @@ template <int MT>
 __global__ __launch_bounds__(256) void head_linear_mfma_kernel(
     const bf16_t* __restrict__ x, long x_stride, int x_head, const bf16_t* __restrict__ W, bf16_t* __restrict__ y,
     long y_stride, int y_head, const bf16_t* __restrict__ gate, long gate_stride, int n_tokens, int O, int K,
-    RopeTailArgs tail) {
+    RopeTailArgs tail, int gate_wide) {
   const int h = blockIdx.y, n0 = blockIdx.x * (16 * MT);
   const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
   const int fr = lane % 16, fg = lane / 16;
@@ -236,11 +241,14 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     if (tok[mt] >= n_tokens) continue;
-    const float g = gate ? 1.f / (1.f + expf(-bf16_to_f32(gate[(long)tok[mt] * gate_stride + h]))) : 1.f;
+    const float g = gate && !gate_wide ? 1.f / (1.f + expf(-bf16_to_f32(gate[(long)tok[mt] * gate_stride + h]))) : 1.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int o = o0 + fg * 4 + j;
-      if (o < O) y[(long)tok[mt] * y_stride + (long)h * y_head + o] = f32_to_bf16(acc[mt][j] * g);
+      if (o >= O) continue;
+      const float gg = gate && gate_wide
+          ? 1.f / (1.f + expf(-bf16_to_f32(gate[(long)tok[mt] * gate_stride + (long)h * O + o]))) : g;
+      y[(long)tok[mt] * y_stride + (long)h * y_head + o] = f32_to_bf16(acc[mt][j] * gg);
     }
   }
 }
@@ -256,7 +264,7 @@ __global__ __launch_bounds__(LAT_THREADS) void rope_tail_kernel(
 extern "C" int lmsf_head_linear(const void* x, int dtype, long x_stride, int x_head, const void* W, void* y,
                                 long y_stride, int y_head, const void* gate, long gate_stride, int n_tokens, int H,
                                 int O, int K, const int* positions, const float* table, int rot, int max_pos, int x_at,
-                                int y_at, int dr, hipStream_t stream) {
+                                int y_at, int dr, int gate_wide, hipStream_t stream) {
   LMSF_CHECK(x && W && y, "head_linear: null pointer");
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "head_linear: unknown dtype code %d", dtype);
   LMSF_CHECK(H > 0 && H <= 65535 && O > 0 && K > 0, "head_linear: bad sizes");
@@ -277,11 +285,11 @@ extern "C" int lmsf_head_linear(const void* x, int dtype, long x_stride, int x_h
     if (n_tokens <= 32 || (long)((n_tokens + 63) / 64) * H * ((O + 63) / 64) < 512)
       hipLaunchKernelGGL(head_linear_mfma_kernel<1>, dim3((n_tokens + 15) / 16, H, (O + 63) / 64), dim3(256), 0, stream,
                          (const bf16_t*)x, x_stride, x_head, (const bf16_t*)W, (bf16_t*)y, y_stride, y_head,
-                         (const bf16_t*)gate, gate_stride, n_tokens, O, K, tail);
+                         (const bf16_t*)gate, gate_stride, n_tokens, O, K, tail, gate_wide);
     else
       hipLaunchKernelGGL(head_linear_mfma_kernel<4>, dim3((n_tokens + 63) / 64, H, (O + 63) / 64), dim3(256), 0, stream,
                          (const bf16_t*)x, x_stride, x_head, (const bf16_t*)W, (bf16_t*)y, y_stride, y_head,
-                         (const bf16_t*)gate, gate_stride, n_tokens, O, K, tail);
+                         (const bf16_t*)gate, gate_stride, n_tokens, O, K, tail, gate_wide);
     LMSF_LAUNCH_CHECK("head_linear (matrix cores)");
     return 0;
   }
@@ -291,14 +299,14 @@ extern "C" int lmsf_head_linear(const void* x, int dtype, long x_stride, int x_h
   if (dtype == LMSF_F32) {
     hipLaunchKernelGGL((head_linear_kernel<float>), grid, dim3(LAT_THREADS), smem, stream, (const float*)x, x_stride,
                        x_head, (const float*)W, (float*)y, y_stride, y_head, (const float*)gate, gate_stride, n_tokens,
-                       O, K, vec);
+                       O, K, vec, gate_wide);
     if (positions)
       hipLaunchKernelGGL((rope_tail_kernel<float>), dim3(n_tokens), dim3(LAT_THREADS), 0, stream, (const float*)x,
                          x_stride, x_head, x_at, (float*)y, y_stride, y_head, y_at, positions, table, rot, max_pos, H, dr);
   } else {
     hipLaunchKernelGGL((head_linear_kernel<bf16_t>), grid, dim3(LAT_THREADS), smem, stream, (const bf16_t*)x, x_stride,
                        x_head, (const bf16_t*)W, (bf16_t*)y, y_stride, y_head, (const bf16_t*)gate, gate_stride,
-                       n_tokens, O, K, vec);
+                       n_tokens, O, K, vec, gate_wide);
     if (positions)
       hipLaunchKernelGGL((rope_tail_kernel<bf16_t>), dim3(n_tokens), dim3(LAT_THREADS), 0, stream, (const bf16_t*)x,
                          x_stride, x_head, x_at, (bf16_t*)y, y_stride, y_head, y_at, positions, table, rot, max_pos, H, dr);

@@ -12,6 +12,11 @@
 // and the up rows of the same outputs), operands through LDS. The down product leaves float32 rows per pair; a last kernel adds a token's pairs and the shared part. A pair's result
 // does not depend on where in its tile it lies, so the order inside an expert's group (atomic counters) is free.
 // Accumulation in float32 throughout.
+//
+// The same kernels serve experts that a router chooses: ``ids`` null makes row n of the table token n's own choice (a
+// table [n_tokens, top] that a kernel of the step has just written, lmsf_moe_route below); ``pair_scale`` gives every
+// (token, choice) a float32 factor on the expert's *input*, y_e(s h), which the gate and up products take as a factor on
+// their results before these are rounded (W (s h) = s (W h)); ``base_scale`` a float32 factor per token on ``base``.
 #include "common.h"
 
 #include <math.h>
@@ -57,12 +62,14 @@ __device__ __forceinline__ void moe_rows_dot(const T* __restrict__ w, long ld, i
 template <typename T>
 __global__ __launch_bounds__(MOE_THREADS) void moe_gate_up_kernel(
     const T* __restrict__ h, long h_stride, const T* __restrict__ Wgu, const int* __restrict__ ids,
-    const int* __restrict__ table, int vocab, int top, int E, T* __restrict__ act, int F, int W, int vec) {
+    const int* __restrict__ table, int vocab, int top, int E, T* __restrict__ act, int F, int W, int vec,
+    const float* __restrict__ pair_scale) {
   extern __shared__ float sh[];   // [W]
   const int nk = blockIdx.x, n = nk / top, k = nk - n * top;
-  const int id = min(max(ids[n], 0), vocab - 1);
+  const int id = min(max(ids ? ids[n] : n, 0), vocab - 1);
   const int e = min(max(table[(long)id * top + k], 0), E - 1);
-  for (int i = threadIdx.x; i < W; i += MOE_THREADS) sh[i] = to_f32<T>(h[(long)n * h_stride + i]);
+  const float ps = pair_scale ? pair_scale[nk] : 1.f;
+  for (int i = threadIdx.x; i < W; i += MOE_THREADS) sh[i] = ps * to_f32<T>(h[(long)n * h_stride + i]);
   __syncthreads();
   const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
   const int f0 = (blockIdx.y * MOE_WAVES + wave) * MOE_OUT_PER_WAVE;
@@ -90,10 +97,10 @@ template <typename T>
 __global__ __launch_bounds__(MOE_THREADS) void moe_down_kernel(
     const T* __restrict__ act, const T* __restrict__ Wd, const int* __restrict__ ids, const int* __restrict__ table,
     int vocab, int top, int E, float weight, const T* __restrict__ base, long base_stride, T* __restrict__ out,
-    long out_stride, int F, int W, int vec) {
+    long out_stride, int F, int W, int vec, const float* __restrict__ base_scale) {
   extern __shared__ float sa[];   // [top, F]
   const int n = blockIdx.x;
-  const int id = min(max(ids[n], 0), vocab - 1);
+  const int id = min(max(ids ? ids[n] : n, 0), vocab - 1);
   for (int i = threadIdx.x; i < top * F; i += MOE_THREADS) sa[i] = to_f32<T>(act[(long)n * top * F + i]);
   __syncthreads();
   const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
@@ -115,7 +122,8 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_down_kernel(
 #pragma unroll
     for (int r = 0; r < MOE_OUT_PER_WAVE; ++r)
       if (r == lane) mine = total[r];
-    const float b = base ? to_f32<T>(base[(long)n * base_stride + o0 + lane]) : 0.f;
+    float b = base ? to_f32<T>(base[(long)n * base_stride + o0 + lane]) : 0.f;
+    if (base_scale) b *= base_scale[n];
     out[(long)n * out_stride + o0 + lane] = from_f32<T>(b + weight * mine);
   }
 }
@@ -138,7 +146,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
   for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = fill[e] = 0;
   __syncthreads();
   for (int p = threadIdx.x; p < P; p += blockDim.x) {
-    const int id = min(max(ids[p / top], 0), vocab - 1);
+    const int id = min(max(ids ? ids[p / top] : p / top, 0), vocab - 1);
     atomicAdd(&cnt[min(max(table[(long)id * top + p % top], 0), E - 1)], 1);
   }
   __syncthreads();
@@ -158,7 +166,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
   }
   __syncthreads();
   for (int p = threadIdx.x; p < P; p += blockDim.x) {
-    const int id = min(max(ids[p / top], 0), vocab - 1);
+    const int id = min(max(ids ? ids[p / top] : p / top, 0), vocab - 1);
     const int e = min(max(table[(long)id * top + p % top], 0), E - 1);
     order[first[e] + atomicAdd(&fill[e], 1)] = p;
   }
@@ -178,7 +186,8 @@ template <bool GATED>
 __global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restrict__ x, long x_stride, int top,
                                                            const bf16_t* __restrict__ Wm, const int* __restrict__ order,
                                                            const int* __restrict__ tiles, const int* __restrict__ n_tiles,
-                                                           void* __restrict__ y, int O, int K) {
+                                                           void* __restrict__ y, int O, int K,
+                                                           const float* __restrict__ pair_scale) {
   constexpr int AR = GATED ? 256 : 128;            // rows of W a step
   constexpr int NLA = AR * 4 / 256;                // 16-byte pieces of W a thread copies a step
   constexpr int NLB = MOE_TILE * 4 / 256;      // and of the pairs' rows
@@ -261,6 +270,7 @@ __global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restr
     const int slot = wr * 64 + mt * 16 + fr;
     if (slot >= count) continue;
     const int p = order[place + slot];
+    const float ps = GATED && pair_scale ? pair_scale[p] : 1.f;
 #pragma unroll
     for (int a = 0; a < 4; ++a)
 #pragma unroll
@@ -268,7 +278,7 @@ __global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restr
         const int o = o_base + wc * 64 + a * 16 + fg * 4 + j;
         if (o >= O) continue;
         if (GATED) {
-          const float g = bf16_to_f32(f32_to_bf16(acc[a][mt][j])), u = bf16_to_f32(f32_to_bf16(acc[NA - 4 + a][mt][j]));
+          const float g = bf16_to_f32(f32_to_bf16(ps * acc[a][mt][j])), u = bf16_to_f32(f32_to_bf16(ps * acc[NA - 4 + a][mt][j]));
           reinterpret_cast<bf16_t*>(y)[(long)p * O + o] = f32_to_bf16(g / (1.f + expf(-g)) * u);
         } else {
           reinterpret_cast<float*>(y)[(long)p * O + o] = acc[a][mt][j];
@@ -280,12 +290,14 @@ __global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restr
 // out[n, o] = base[n, o] + weight * sum_k rows[n * top + k, o]
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ rows, int top, float weight,
                                                           const bf16_t* __restrict__ base, long base_stride,
-                                                          bf16_t* __restrict__ out, long out_stride, int W) {
+                                                          bf16_t* __restrict__ out, long out_stride, int W,
+                                                          const float* __restrict__ base_scale) {
   const int n = blockIdx.x;
+  const float bs = base_scale ? base_scale[n] : 1.f;
   for (int o = threadIdx.x; o < W; o += 256) {
     float s = 0.f;
     for (int k = 0; k < top; ++k) s += rows[((long)n * top + k) * W + o];
-    const float b = base ? bf16_to_f32(base[(long)n * base_stride + o]) : 0.f;
+    const float b = base ? bs * bf16_to_f32(base[(long)n * base_stride + o]) : 0.f;
     out[(long)n * out_stride + o] = f32_to_bf16(b + weight * s);
   }
 }
@@ -305,9 +317,11 @@ extern "C" int lmsf_table_moe_grouped(int dtype, int n_tokens, int top, int E, i
 
 extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const void* Wgu, const void* Wd, const int* ids,
                               const int* table, int vocab, int top, int E, float weight, const void* base,
-                              long base_stride, void* act, void* out, long out_stride, int n_tokens, int F, int W,
-                              int* scratch_ints, float* scratch_rows, hipStream_t stream) {
-  LMSF_CHECK(h && Wgu && Wd && ids && table && act && out, "table_moe: null pointer");
+                              long base_stride, const float* pair_scale, const float* base_scale, void* act, void* out,
+                              long out_stride, int n_tokens, int F, int W, int* scratch_ints, float* scratch_rows,
+                              hipStream_t stream) {
+  LMSF_CHECK(h && Wgu && Wd && table && act && out, "table_moe: null pointer");
+  LMSF_CHECK(ids || vocab >= n_tokens, "table_moe: without token ids the table has a row per token");
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "table_moe: unknown dtype code %d", dtype);
   LMSF_CHECK(vocab > 0 && top > 0 && E > 0 && F > 0 && W > 0, "table_moe: bad sizes");
   LMSF_CHECK(h_stride >= W && out_stride >= W && (!base || base_stride >= W), "table_moe: rows overlap");
@@ -323,12 +337,12 @@ extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const voi
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)3 * E * 4, stream, ids, table, vocab, top, E, P,
                        MOE_TILE, order, tiles, n_tiles);
     hipLaunchKernelGGL((moe_tile_lds_kernel<true>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream,
-                       (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
+                       (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W, pair_scale);
     hipLaunchKernelGGL((moe_tile_lds_kernel<false>), dim3(max_tiles, (W + 127) / 128), dim3(256), 0, stream,
                        (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows, W,
-                       F);
+                       F, (const float*)nullptr);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(256), 0, stream, scratch_rows, top, weight,
-                       (const bf16_t*)base, base_stride, (bf16_t*)out, out_stride, W);
+                       (const bf16_t*)base, base_stride, (bf16_t*)out, out_stride, W, base_scale);
     LMSF_LAUNCH_CHECK("table_moe (grouped)");
     return 0;
   }
@@ -338,17 +352,78 @@ extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const voi
   const int vec1 = W % vn == 0 && lmsf_aligned16(Wgu), vec2 = F % vn == 0 && lmsf_aligned16(Wd);
   if (dtype == LMSF_F32) {
     hipLaunchKernelGGL((moe_gate_up_kernel<float>), g1, dim3(MOE_THREADS), (size_t)W * 4, stream, (const float*)h,
-                       h_stride, (const float*)Wgu, ids, table, vocab, top, E, (float*)act, F, W, vec1);
+                       h_stride, (const float*)Wgu, ids, table, vocab, top, E, (float*)act, F, W, vec1, pair_scale);
     hipLaunchKernelGGL((moe_down_kernel<float>), g2, dim3(MOE_THREADS), (size_t)top * F * 4, stream, (const float*)act,
                        (const float*)Wd, ids, table, vocab, top, E, weight, (const float*)base, base_stride,
-                       (float*)out, out_stride, F, W, vec2);
+                       (float*)out, out_stride, F, W, vec2, base_scale);
   } else {
     hipLaunchKernelGGL((moe_gate_up_kernel<bf16_t>), g1, dim3(MOE_THREADS), (size_t)W * 4, stream, (const bf16_t*)h,
-                       h_stride, (const bf16_t*)Wgu, ids, table, vocab, top, E, (bf16_t*)act, F, W, vec1);
+                       h_stride, (const bf16_t*)Wgu, ids, table, vocab, top, E, (bf16_t*)act, F, W, vec1, pair_scale);
     hipLaunchKernelGGL((moe_down_kernel<bf16_t>), g2, dim3(MOE_THREADS), (size_t)top * F * 4, stream,
                        (const bf16_t*)act, (const bf16_t*)Wd, ids, table, vocab, top, E, weight, (const bf16_t*)base,
-                       base_stride, (bf16_t*)out, out_stride, F, W, vec2);
+                       base_stride, (bf16_t*)out, out_stride, F, W, vec2, base_scale);
   }
   LMSF_LAUNCH_CHECK("table_moe");
+  return 0;
+}
+
+// ---------------------------------------------------------------- a router's choice
+// From float32 router logits z [n_tokens, >= E]: scores s = sigmoid(z); choice[n, 0 .. top-1] the experts with the
+// largest scores (the largest first; of equal scores the lower index), weight[n, k] their scores, divided by their sum
+// if ``renorm``. ``extra`` >= 0: also gate[n] = sigmoid(z[n, extra]) (a column beside the experts': the gate of a
+// shared expert). A wave a token; top times a pass over the E scores.
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ z, long z_stride, int n_tokens, int E,
+                                                        int top, int renorm, int extra, int* __restrict__ choice,
+                                                        float* __restrict__ weight, float* __restrict__ gate) {
+  const int n = blockIdx.x * (256 / LMSF_WAVE) + threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
+  if (n >= n_tokens) return;
+  const float* row = z + (long)n * z_stride;
+  float last = INFINITY, total = 0.f, mine = 0.f;
+  int last_e = -1, mine_e = 0;
+  for (int k = 0; k < top; ++k) {
+    // the largest (score, -index) below the one taken before
+    float best = -INFINITY;
+    int best_e = E;
+    for (int e = lane; e < E; e += LMSF_WAVE) {
+      const float sc = row[e];
+      const bool below = sc < last || (sc == last && e > last_e);
+      if (below && (sc > best || (sc == best && e < best_e))) {
+        best = sc;
+        best_e = e;
+      }
+    }
+#pragma unroll
+    for (int o = LMSF_WAVE / 2; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, LMSF_WAVE);
+      const int oe = __shfl_xor(best_e, o, LMSF_WAVE);
+      if (ob > best || (ob == best && oe < best_e)) {
+        best = ob;
+        best_e = oe;
+      }
+    }
+    last = best;
+    last_e = best_e;
+    const float sg = 1.f / (1.f + expf(-best));
+    total += sg;
+    if (lane == k) {      // lane k keeps the k-th choice
+      mine = sg;
+      mine_e = min(best_e, E - 1);
+    }
+  }
+  if (lane < top) {
+    choice[(long)n * top + lane] = mine_e;
+    weight[(long)n * top + lane] = renorm ? mine / total : mine;
+  }
+  if (extra >= 0 && lane == 0) gate[n] = 1.f / (1.f + expf(-row[extra]));
+}
+
+extern "C" int lmsf_moe_route(const float* z, long z_stride, int n_tokens, int E, int top, int renorm, int extra,
+                              int* choice, float* weight, float* gate, hipStream_t stream) {
+  LMSF_CHECK(z && choice && weight && (extra < 0 || gate), "moe_route: null pointer");
+  LMSF_CHECK(E > 0 && top > 0 && top <= E && top <= LMSF_WAVE && z_stride >= E && extra < z_stride, "moe_route: bad sizes");
+  if (n_tokens <= 0) return 0;
+  hipLaunchKernelGGL(moe_route_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, stream, z, z_stride, n_tokens, E, top,
+                     renorm, extra, choice, weight, gate);
+  LMSF_LAUNCH_CHECK("moe_route");
   return 0;
 }

@@ -673,9 +673,10 @@ class HipOps:
         return q_out
 
     def head_linear(self, x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.Tensor, out_head: int,
-                    gate: Optional[torch.Tensor] = None, rope_tail=None) -> torch.Tensor:
+                    gate: Optional[torch.Tensor] = None, rope_tail=None, gate_wide: bool = False) -> torch.Tensor:
         """Per-head products: out[n, h * out_head + o] = sum_k weight[h, o, k] x[n, h * x_head + k], times
-        sigmoid(gate[n, h]) if a gate is given. ``weight`` contiguous [H, O, K]; x, out and gate are views with
+        sigmoid(gate[n, h]) if a gate is given (``gate_wide``: a gate per output, sigmoid(gate[n, h * O + o])).
+        ``weight`` contiguous [H, O, K]; x, out and gate are views with
         unit column stride whose first column is head 0's first entry. ``rope_tail`` = (x_at, out_at, width,
         positions, table): also what ``rope_tail`` does with these arguments, from the same launch where it can be."""
         self._dev(x, weight, out, gate)
@@ -695,12 +696,13 @@ class HipOps:
         if x.stride(1) != 1 or out.stride(1) != 1 or x.shape[1] < (H - 1) * x_head + K \
                 or out.shape[1] < (H - 1) * out_head + O or out.shape[0] != N:
             raise ValueError("head_linear: operands too narrow for %d heads" % H)
-        if gate is not None and (gate.dtype != x.dtype or gate.stride(1) != 1 or gate.shape[1] < H or gate.shape[0] != N):
-            raise ValueError("head_linear: gate must be [N, >= %d] of x's dtype" % H)
+        need = H * O if gate_wide else H
+        if gate is not None and (gate.dtype != x.dtype or gate.stride(1) != 1 or gate.shape[1] < need or gate.shape[0] != N):
+            raise ValueError("head_linear: gate must be [N, >= %d] of x's dtype" % need)
         self._check(self.lib.lmsf_head_linear(
             _ptr(x), _code(x.dtype), x.stride(0), int(x_head), _ptr(weight), _ptr(out), out.stride(0), int(out_head),
             _ptr(gate), gate.stride(0) if gate is not None else 0, N, H, O, K, _ptr(positions), _ptr(table), rot, max_pos,
-            int(x_at), int(out_at), int(width), self._stream()))
+            int(x_at), int(out_at), int(width), 1 if (gate_wide and gate is not None) else 0, self._stream()))
         return out
 
     def rope_tail(self, x: torch.Tensor, x_head: int, x_at: int, out: torch.Tensor, out_head: int, out_at: int,
@@ -721,11 +723,15 @@ class HipOps:
             int(out_at), _ptr(positions), _ptr(table), table.shape[1], table.shape[0], N, int(heads), int(width),
             self._stream()))
 
-    def table_moe(self, h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, token_ids: torch.Tensor,
-                  table: torch.Tensor, weight: float, base: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def table_moe(self, h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, token_ids: Optional[torch.Tensor],
+                  table: torch.Tensor, weight: float, base: Optional[torch.Tensor] = None,
+                  pair_scale: Optional[torch.Tensor] = None, base_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
         """out[n] = base[n] + weight * sum_k down_e(silu(gate_e h[n]) * up_e h[n]) over e = table[token_ids[n], k].
-        ``w_gate_up`` [E, 2 F, W] (gate rows first), ``w_down`` [E, W, F], ``table`` int32 [vocab, top]."""
-        self._dev(h, w_gate_up, w_down, token_ids, table, base)
+        ``w_gate_up`` [E, 2 F, W] (gate rows first), ``w_down`` [E, W, F], ``table`` int32 [vocab, top].
+        ``token_ids`` None: row n of the table is token n's choice (a router's, ``moe_route``). ``pair_scale``
+        (float32 [N, top]): the expert of (n, k) gets pair_scale[n, k] * h[n] as its input. ``base_scale``
+        (float32 [N]): base[n] is multiplied by it."""
+        self._dev(h, w_gate_up, w_down, token_ids, table, base, pair_scale, base_scale)
         N, W = h.shape
         E, F2, _ = w_gate_up.shape
         F = F2 // 2
@@ -738,6 +744,14 @@ class HipOps:
         if table.dtype != torch.int32 or table.dim() != 2 or not table.is_contiguous():
             raise ValueError("table_moe: table must be contiguous int32 [vocab, top]")
         vocab, top = table.shape
+        if token_ids is None and vocab < N:
+            raise ValueError("table_moe: without token ids the table needs a row per token")
+        if pair_scale is not None and (pair_scale.dtype != torch.float32 or pair_scale.numel() != N * top
+                                       or not pair_scale.is_contiguous()):
+            raise ValueError("table_moe: pair_scale must be contiguous float32 [%d, %d]" % (N, top))
+        if base_scale is not None and (base is None or base_scale.dtype != torch.float32 or base_scale.numel() != N
+                                       or not base_scale.is_contiguous()):
+            raise ValueError("table_moe: base_scale must be contiguous float32 [%d] beside a base" % N)
         act = torch.empty((N * top, F), dtype=h.dtype, device=h.device)
         out = torch.empty((N, W), dtype=h.dtype, device=h.device)
         ints = rows = None
@@ -747,8 +761,129 @@ class HipOps:
             rows = torch.empty((N * top, W), dtype=torch.float32, device=h.device)
         self._check(self.lib.lmsf_table_moe(
             _ptr(h), _code(h.dtype), h.stride(0), _ptr(w_gate_up), _ptr(w_down), _ptr(token_ids), _ptr(table), vocab,
-            top, E, float(weight), _ptr(base), base.stride(0) if base is not None else 0, _ptr(act), _ptr(out),
-            out.stride(0), N, F, W, _ptr(ints), _ptr(rows), self._stream()))
+            top, E, float(weight), _ptr(base), base.stride(0) if base is not None else 0, _ptr(pair_scale),
+            _ptr(base_scale), _ptr(act), _ptr(out), out.stride(0), N, F, W, _ptr(ints), _ptr(rows), self._stream()))
+        return out
+
+    def moe_route(self, logits: torch.Tensor, experts: int, top: int, renorm: bool = False, extra: int = -1):
+        """A router's choice from float32 logits [N, >= experts]: (choice int32 [N, top], weight float32 [N, top],
+        gate float32 [N] or None). Scores are sigmoid(logits); the ``top`` largest choose (the largest first, the
+        lower index among equals); the weights are their scores, divided by their sum with ``renorm``. ``extra``
+        >= 0 names a column beside the experts' whose sigmoid is returned as ``gate``."""
+        self._dev(logits)
+        if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1 or logits.shape[1] < experts \
+                or extra >= logits.shape[1]:
+            raise ValueError("moe_route: logits must be float32 [N, >= %d] with unit column stride" % experts)
+        if not (0 < top <= experts and top <= 64):
+            raise ValueError("moe_route: %d of %d experts (at most 64 a token)" % (top, experts))
+        N = logits.shape[0]
+        choice = torch.empty((N, top), dtype=torch.int32, device=logits.device)
+        weight = torch.empty((N, top), dtype=torch.float32, device=logits.device)
+        gate = torch.empty((N,), dtype=torch.float32, device=logits.device) if extra >= 0 else None
+        self._check(self.lib.lmsf_moe_route(_ptr(logits), logits.stride(0), N, int(experts), int(top), 1 if renorm else 0,
+                                            int(extra), _ptr(choice), _ptr(weight), _ptr(gate), self._stream()))
+        return choice, weight, gate
+
+    # ------------------------------------------------------------------ layer scale, logit cap
+
+    def scale_add_norm(self, a: torch.Tensor, scale_a: torch.Tensor, b: Optional[torch.Tensor],
+                       scale_b: Optional[torch.Tensor], residual: torch.Tensor, weight: Optional[torch.Tensor] = None,
+                       eps: float = 1e-5) -> Optional[torch.Tensor]:
+        """residual += scale_a * a + scale_b * b (float32, in place; b may be None), and with ``weight`` the RMS norm
+        of the new rows times ``weight`` in a's dtype, from the same launch. a, b [N, W] with unit column stride;
+        the scales float32 [W]; residual contiguous float32 [N, W]."""
+        self._dev(a, scale_a, b, scale_b, residual, weight)
+        if a.dim() != 2 or a.stride(1) != 1 or residual.dtype != torch.float32 or not residual.is_contiguous() \
+                or residual.shape != a.shape:
+            raise ValueError("scale_add_norm: a [N, W] and a contiguous float32 stream of that shape are needed")
+        N, W = a.shape
+        self._f32_vec(scale_a, W, "scale_add_norm: first scale")
+        if b is not None:
+            if b.shape != a.shape or b.dtype != a.dtype or b.stride(1) != 1 or scale_b is None:
+                raise ValueError("scale_add_norm: b must be like a and have its scale")
+            self._f32_vec(scale_b, W, "scale_add_norm: second scale")
+        out = None
+        if weight is not None:
+            if weight.shape != (W,) or not weight.is_contiguous():
+                raise ValueError("scale_add_norm: the norm's weight must be [%d]" % W)
+            out = torch.empty((N, W), dtype=a.dtype, device=a.device)
+        self._check(self.lib.lmsf_scale_add_norm(
+            _ptr(a), a.stride(0), _ptr(scale_a), _ptr(b), b.stride(0) if b is not None else 0, _ptr(scale_b),
+            _code(a.dtype), _ptr(residual), _ptr(weight), _code(weight.dtype) if weight is not None else F32, _ptr(out),
+            N, W, float(eps), self._stream()))
+        return out
+
+    def logit_cap(self, logits: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> torch.Tensor:
+        """logits <- cap tanh(logits * scale / cap) (cap 0: logits * scale), float32 [R, V], in place."""
+        self._dev(logits)
+        if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+            raise ValueError("logit_cap: logits must be float32 [R, V] with unit column stride")
+        R, V = logits.shape
+        for r0 in range(0, R, 65535):
+            part = logits[r0:r0 + 65535]
+            self._check(self.lib.lmsf_logit_cap(_ptr(part), part.stride(0), part.shape[0], V, float(scale), float(cap),
+                                                self._stream()))
+        return logits
+
+    # ------------------------------------------------------------------ retention
+
+    def retention_state_floats(self, heads: int, dim: int, vdim: int) -> int:
+        return int(self.lib.lmsf_retention_state_floats(heads, dim, vdim))
+
+    def retention(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, out_gate: torch.Tensor,
+                  state: torch.Tensor, batch, heads: int, dim: int, vdim: int, q_scale: float, eps: float,
+                  table: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Linear attention with a fixed decay per head over each request's tokens, the memory S [heads, dim, vdim]
+        carried in ``state`` (float32 [slots, >= heads * dim * vdim]): S <- decay S + k v^T, o = S^T (q * q_scale);
+        returns every head's o over its root mean square times silu(out_gate), [N, heads * vdim] in q's dtype.
+        q, k [N, heads * dim] and v [N, heads * vdim]: views of one buffer (equal row strides). ``decay``: float32
+        [2 heads], the decays and then their logarithms. ``table`` (float32 [max_pos, rot] = [cos | sin]): q and k
+        are first rotated by the token's position over their first rot entries, pairs (i, i + rot/2)."""
+        self._dev(q, k, v, decay, out_gate, table)
+        N = q.shape[0]
+        for t, w, name in ((q, heads * dim, "q"), (k, heads * dim, "k"), (v, heads * vdim, "v"),
+                           (out_gate, heads * vdim, "out_gate")):
+            if t.dim() != 2 or t.shape[0] != N or t.shape[1] < w or t.stride(1) != 1 or t.dtype != q.dtype:
+                raise ValueError("retention: %s must be [%d, >= %d] of q's dtype with unit column stride" % (name, N, w))
+        if not (q.stride(0) == k.stride(0) == v.stride(0)):
+            raise ValueError("retention: q, k and v must have one row stride")
+        self._f32_vec(decay, 2 * heads, "retention: decay")
+        rot = max_pos = 0
+        if table is not None:
+            if table.dtype != torch.float32 or table.dim() != 2 or not table.is_contiguous() or table.shape[1] > dim \
+                    or table.shape[1] % 2:
+                raise ValueError("retention: the rotary table must be contiguous float32 [max_pos, rot <= %d]" % dim)
+            max_pos, rot = table.shape
+            self._i32(batch.positions, "positions", N)
+            self._dev(batch.positions)
+        self._state_view(state, self.retention_state_floats(heads, dim, vdim), "retention")
+        _, seg_starts, slots, S = self._segments(batch, N)
+        out = torch.empty((N, heads * vdim), dtype=q.dtype, device=q.device)
+        raw = torch.empty((N, heads * vdim), dtype=torch.float32, device=q.device)
+        head = (_ptr(q), _ptr(k), _ptr(v), _code(q.dtype), q.stride(0), _ptr(batch.positions) if table is not None else None,
+                _ptr(table), rot, max_pos, _ptr(decay), _ptr(out_gate), out_gate.stride(0), _ptr(state), state.stride(0),
+                _ptr(seg_starts), _ptr(slots), _ptr(out), out.stride(0), _ptr(raw), N, S, int(heads), int(dim), int(vdim),
+                float(q_scale), float(eps))
+        lens = getattr(batch, "host_seg_lens", None)
+        L = self.lib.lmsf_retention_chunk_tokens(int(dim))
+        if not getattr(batch, "replayed", False) and not getattr(batch, "all_single", False) and lens and L > 0 \
+                and max(lens) >= self.recurrent_chunked_min_tokens:
+            bases = entries = None
+            n_entries, most = 0, 1
+            if max(lens) >= self.recurrent_parallel_min_chunks * L:
+                key = ("retention_chunks", L)
+                plan = batch.aux.get(key)
+                if plan is None:
+                    counts = [-(-n // L) for n in lens]
+                    firsts = [sum(counts[:i]) for i in range(len(counts))]
+                    plan = batch.aux[key] = (self.upload_ints(firsts, q.device), sum(counts), max(counts))
+                bases, n_entries, most = plan
+                entries = torch.empty(n_entries * self.lib.lmsf_retention_chunk_entry_floats(heads, dim, vdim),
+                                      dtype=torch.float32, device=q.device)
+            self._check(self.lib.lmsf_retention_chunked(*head, _ptr(bases), int(most), int(n_entries), _ptr(entries),
+                                                        self._stream()))
+            return out
+        self._check(self.lib.lmsf_retention_tokens(*head, self._stream()))
         return out
 
     # ------------------------------------------------------------------ Dynamic Tanh, state-carrying mixers

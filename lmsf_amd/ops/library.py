@@ -10,7 +10,7 @@ from typing import Optional
 from ..csrc import build as _build
 from .dispatch import ProductShape, Route, Tunables
 
-ABI_VERSION = 28
+ABI_VERSION = 29
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -44,11 +44,22 @@ _SIGNATURES = {
     "lmsf_latent_cache_write": (c_int, [_P, c_int, c_long, _P, c_float, _P, _P, c_int, c_int, _P, _P, _P, c_long, c_int,
                                         c_int, c_int, c_int, c_int, _P, _P, _P, c_long, c_int, _P]),
     "lmsf_head_linear": (c_int, [_P, c_int, c_long, c_int, _P, _P, c_long, c_int, _P, c_long, c_int, c_int, c_int, c_int,
-                                 _P, _P, c_int, c_int, c_int, c_int, c_int, _P]),
+                                 _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, _P]),
     "lmsf_rope_tail": (c_int, [_P, c_int, c_long, c_int, c_int, _P, c_long, c_int, c_int, _P, _P, c_int, c_int, c_int,
                                c_int, c_int, _P]),
-    "lmsf_table_moe": (c_int, [_P, c_int, c_long, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, c_long, _P, _P,
+    "lmsf_table_moe": (c_int, [_P, c_int, c_long, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, c_long, _P, _P, _P, _P,
                                c_long, c_int, c_int, c_int, _P, _P, _P]),
+    "lmsf_moe_route": (c_int, [_P, c_long, c_int, c_int, c_int, c_int, c_int, _P, _P, _P, _P]),
+    "lmsf_retention_state_floats": (c_long, [c_int, c_int, c_int]),
+    "lmsf_retention_chunk_tokens": (c_int, [c_int]),
+    "lmsf_retention_chunk_entry_floats": (c_long, [c_int, c_int, c_int]),
+    "lmsf_retention_chunked": (c_int, [_P, _P, _P, c_int, c_long, _P, _P, c_int, c_int, _P, _P, c_long, _P, c_long, _P, _P,
+                                       _P, c_long, _P, c_int, c_int, c_int, c_int, c_int, c_float, c_float, _P, c_int,
+                                       c_long, _P, _P]),
+    "lmsf_retention_tokens": (c_int, [_P, _P, _P, c_int, c_long, _P, _P, c_int, c_int, _P, _P, c_long, _P, c_long, _P, _P,
+                                      _P, c_long, _P, c_int, c_int, c_int, c_int, c_int, c_float, c_float, _P]),
+    "lmsf_scale_add_norm": (c_int, [_P, c_long, _P, _P, c_long, _P, c_int, _P, _P, c_int, _P, c_int, c_int, c_float, _P]),
+    "lmsf_logit_cap": (c_int, [_P, c_long, c_int, c_int, c_float, c_float, _P]),
     "lmsf_table_moe_scratch_ints": (c_long, [c_int, c_int, c_int]),
     "lmsf_table_moe_grouped": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_long]),
     "lmsf_dyt_norm": (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P]),

@@ -3,7 +3,7 @@ from .base import (Block, CacheBinding, CacheSpec, FeedForward, LayerSpec, Mixer
                    PartSpec, PositionEncoding, Runtime, ScheduleEntry, StateSpec, TensorDecl, build_part,
                    part_class, register_part, unregister_part)
 from . import (attention, block, dyt_norm, embedding, flex_attention, group_norm, latent_attention,  # noqa: F401  (registration)
-               mlp, norm, parallel, recurrent, rotary, table_moe)
+               mlp, norm, parallel, recurrent, retention, rotary, routed_moe, table_moe)
 from .linear import FusedLinear, Linear
 
 __all__ = ["Block", "CacheBinding", "CacheSpec", "FeedForward", "LayerSpec", "Mixer", "ModelSpec", "Norm", "Part",

@@ -132,3 +132,68 @@ class SandwichDepthBlock(Block):
             ahead = norm.add_normed(branch, residual, then=self.next_norm, history=hist, index=self.depth, mix=mix)
         if ahead is not None:
             ctx.aux["prenormed"] = ahead
+
+
+@register_part("block", "parallel_scaled")
+class ParallelScaledBlock(Block):
+    """One norm, two sublayers that both read it, each result scaled entry by entry before the sum:
+
+        h = norm(x);   x += scale_mixer * mixer(h) + scale_ffn * ffn(h)
+
+    (without a feed-forward only the first term). The scales are checkpoint vectors of the layer, float32, as are
+    the stream and the sum. The addition and the norm that the next block begins with are one kernel where the
+    model has linked the blocks (``link_next``); nothing is left to add when the block returns. The reference's
+    only arrangement is the pre-norm one with two norms (core/src/model_executor/models/llama/llama.rs:286-340).
+    """
+
+    graph_safe = True
+    recordable = False
+
+    ROLES = ("input",)
+
+    def __init__(self, prefix: str, rt: Runtime, mixer, feed_forward, norms, hidden_size: int,
+                 mixer_scale_name: str = "ls1", ffn_scale_name: str = "ls2"):
+        super().__init__(prefix, rt, mixer, feed_forward, norms)
+        self.has_ffn = not getattr(feed_forward, "absent", False)
+        self.W = int(hidden_size)
+        self.names = ("%s.%s" % (prefix, mixer_scale_name), "%s.%s" % (prefix, ffn_scale_name))
+        self.mixer_scale: Optional[torch.Tensor] = None
+        self.ffn_scale: Optional[torch.Tensor] = None
+        self.next_norm = None
+
+    def link_next(self, following: Block) -> None:
+        """The block that always runs after this one begins with a norm of the stream: this block's closing kernel
+        computes it as well and leaves it in ``ctx.aux["prenormed"]``."""
+        nxt = following.norms.get("input") if isinstance(following, ParallelScaledBlock) else None
+        if nxt is not None and getattr(nxt, "weight_offset", 0.0) == 0.0 and hasattr(nxt, "eps"):
+            self.next_norm = nxt
+
+    def checkpoint_tensors(self):
+        from .base import TensorDecl
+        out = {self.names[0]: TensorDecl((self.W,), init="ones", keeps_float32=True)}
+        if self.has_ffn:
+            out[self.names[1]] = TensorDecl((self.W,), init="ones", keeps_float32=True)
+        return out
+
+    def load_weights(self, fetch) -> None:
+        self.mixer_scale = fetch(self.names[0]).to(torch.float32).contiguous()
+        if self.has_ffn:
+            self.ffn_scale = fetch(self.names[1]).to(torch.float32).contiguous()
+
+    def tensors(self):
+        return [t for t in (self.mixer_scale, self.ffn_scale) if t is not None]
+
+    def forward(self, branch: Optional[torch.Tensor], residual: torch.Tensor, ctx, binding: CacheBinding):
+        norm = self.norms["input"]
+        h = ctx.aux.pop("prenormed", None) if branch is None else None
+        if h is None:
+            h = norm.forward_add(branch, residual)
+        a = self.mixer.forward(h, ctx, binding)
+        f = self.feed_forward.forward(h) if self.has_ffn else None
+        nxt = self.next_norm
+        ahead = self.rt.ops.scale_add_norm(a, self.mixer_scale, f, self.ffn_scale, residual,
+                                           weight=nxt.weight if nxt is not None else None,
+                                           eps=nxt.eps if nxt is not None else 0.0)
+        if ahead is not None:
+            ctx.aux["prenormed"] = ahead
+        return None

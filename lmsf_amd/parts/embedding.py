@@ -39,13 +39,17 @@ class TokenEmbedding(Part):
 @register_part("head", "lm_head")
 class LMHead(Part):
     """``weight_name`` is the full checkpoint name of the [V, H] matrix: the head's own, or the
-    embedding table's when the two are tied (the loader then shares one device tensor)."""
+    embedding table's when the two are tied (the loader then shares one device tensor). ``logit_scale`` multiplies the
+    logits; ``softcap`` c > 0 then bounds them, c tanh(logits / c) (one elementwise kernel behind the product)."""
 
     graph_safe = True
 
     def __init__(self, prefix: str, rt: Runtime, vocab_size: int, hidden_size: int, weight_name: Optional[str] = None,
-                 bias: bool = False):
+                 bias: bool = False, logit_scale: float = 1.0, softcap: float = 0.0):
         super().__init__(prefix, rt)
+        self.logit_scale, self.softcap = float(logit_scale), float(softcap)
+        if self.softcap < 0:
+            raise ValueError("lm_head: softcap must be >= 0")
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.weight_name = weight_name or "%s.weight" % prefix
         self.bias_name = "%s.bias" % prefix if bias else None
@@ -66,5 +70,9 @@ class LMHead(Part):
     def forward(self, h: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """[R, H] -> float32 logits [R, V], written into ``out`` if one is given."""
         if out is not None:
-            return self.rt.ops.linear(h, self.weight, self.bias, out_dtype=torch.float32, out=out)
-        return self.rt.ops.linear(h, self.weight, self.bias, out_dtype=torch.float32)
+            y = self.rt.ops.linear(h, self.weight, self.bias, out_dtype=torch.float32, out=out)
+        else:
+            y = self.rt.ops.linear(h, self.weight, self.bias, out_dtype=torch.float32)
+        if self.logit_scale != 1.0 or self.softcap > 0.0:
+            self.rt.ops.logit_cap(y, self.logit_scale, self.softcap)
+        return y

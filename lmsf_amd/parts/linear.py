@@ -24,8 +24,11 @@ class FusedLinear(Part):
     graph_safe = True
 
     def __init__(self, prefix: str, rt: Runtime, in_features: int, sources: Sequence[Tuple[str, int]],
-                 bias=False, bare_names: bool = False, bias_name: str = "bias"):
+                 bias=False, bare_names: bool = False, bias_name: str = "bias", row_orders=None):
         super().__init__(prefix, rt)
+        # sub-name -> for every row of the loaded source the checkpoint row it holds (a mixer that wants its
+        # outputs in another order than the checkpoint's, e.g. rotation pairs side by side instead of interleaved)
+        self.row_orders = {str(k): [int(i) for i in v] for k, v in (row_orders or {}).items()}
         self.bare_names = bool(bare_names)
         self.bias_name = str(bias_name)
         self.biased = None if isinstance(bias, bool) else set(str(b) for b in bias)   # None: all or none
@@ -82,6 +85,8 @@ class FusedLinear(Part):
                 row += rows
                 continue
             t = fetch(self._name(sub, what))
+            if sub in self.row_orders:
+                t = t[torch.as_tensor(self.row_orders[sub], dtype=torch.long, device=t.device)]
             if (t.dtype != out.dtype and t.dtype == torch.float32) or t.device != out.device:
                 # a source stored in 32 bits: the buffer takes the widest type (and lies where the sources lie)
                 wider = self._buffer(what, torch.float32 if t.dtype == torch.float32 else out.dtype, t.device)
@@ -107,5 +112,6 @@ class Linear(FusedLinear):
     """A single checkpoint matrix ``prefix.name.weight`` [out_features, in_features]."""
 
     def __init__(self, prefix: str, rt: Runtime, name: str, in_features: int, out_features: int, bias: bool = False,
-                 bare_names: bool = False, bias_name: str = "bias"):
-        super().__init__(prefix, rt, in_features, [(name, out_features)], bias, bare_names, bias_name)
+                 bare_names: bool = False, bias_name: str = "bias", row_order=None):
+        super().__init__(prefix, rt, in_features, [(name, out_features)], bias, bare_names, bias_name,
+                         row_orders={name: row_order} if row_order is not None else None)

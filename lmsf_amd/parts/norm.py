@@ -24,7 +24,8 @@ class RMSNorm(Norm):
         self.size = int(size)
         self.eps = float(eps)
         self.weight_offset = float(weight_offset)
-        self.weight_name = "%s.%s" % (prefix, weight_name)
+        # (weight_name "": the weight is the tensor ``prefix`` itself)
+        self.weight_name = "%s.%s" % (prefix, weight_name) if weight_name else prefix
         self.weight: Optional[torch.Tensor] = None
 
     def checkpoint_tensors(self) -> Dict[str, TensorDecl]:

@@ -9,6 +9,12 @@ itself is done by the kernel that also writes the cache.
 rope_scaling "llama3" changes each frequency by its wavelength L = 2 pi / f relative to the
 original context length o: L < o / high_freq_factor keeps f, L > o / low_freq_factor gives
 f / factor, in between (1 - s) f / factor + s f with s = (o / L - low) / (high - low).
+
+rope_scaling "yarn" blends by the pair's index instead: with turn(t) = rot ln(o / (2 pi t)) / (2 ln theta) the index
+at which a pair makes t turns over the original length o, lo = max(floor(turn(beta_fast)), 0),
+hi = min(ceil(turn(beta_slow)), rot - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i gets
+f_i / factor * ramp_i + f_i (1 - ramp_i); and cos and sin are both multiplied by 0.1 ln(factor) + 1
+(``table_gain``), which the table carries.
 """
 import math
 from typing import Any, Callable, Mapping, Optional
@@ -25,8 +31,20 @@ def inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[Mapping
     kind = "default" if not scaling else scaling.get("rope_type", "default")
     if kind == "default":
         return inv
+    if kind == "yarn":
+        factor, orig = float(scaling["factor"]), float(scaling["original_max_position_embeddings"])
+
+        def turn(t: float) -> float:
+            return rotary_dim * math.log(orig / (2.0 * math.pi * t)) / (2.0 * math.log(theta))
+
+        lo = max(math.floor(turn(float(scaling["beta_fast"]))), 0)
+        hi = min(math.ceil(turn(float(scaling["beta_slow"]))), rotary_dim - 1)
+        idx = torch.arange(rotary_dim // 2, dtype=torch.float64)
+        f = torch.pow(torch.tensor(float(theta), dtype=torch.float64), -2.0 * idx / rotary_dim)
+        ramp = torch.clamp((idx - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return (f / factor * ramp + f * (1.0 - ramp)).to(torch.float32)
     if kind != "llama3":
-        raise ValueError("rotary scaling %r is not supported (default, llama3)" % kind)
+        raise ValueError("rotary scaling %r is not supported (default, llama3, yarn)" % kind)
     factor = float(scaling["factor"])
     low, high = float(scaling["low_freq_factor"]), float(scaling["high_freq_factor"])
     orig = float(scaling["original_max_position_embeddings"])
@@ -36,6 +54,13 @@ def inverse_frequencies(rotary_dim: int, theta: float, scaling: Optional[Mapping
     blended = (1.0 - smooth) * f / factor + smooth * f
     scaled = torch.where(wavelength < orig / high, f, torch.where(wavelength > orig / low, f / factor, blended))
     return scaled.to(torch.float32)
+
+
+def table_gain(scaling: Optional[Mapping[str, Any]]) -> float:
+    """What cos and sin are multiplied by: 0.1 ln(factor) + 1 under "yarn" scaling, else 1."""
+    if scaling and scaling.get("rope_type") == "yarn":
+        return 0.1 * math.log(float(scaling["factor"])) + 1.0
+    return 1.0
 
 
 @register_part("position", "rotary")
@@ -70,6 +95,9 @@ class RotaryEncoding(PositionEncoding):
             pos = torch.arange(self.rt.max_positions, dtype=torch.float32)
             angles = pos[:, None] * inv[None, :]
             table = torch.cat([torch.cos(angles), torch.sin(angles)], dim=1).contiguous()
+            gain = table_gain(self.scaling)
+            if gain != 1.0:
+                table = table * gain
             self.rt.shared[key] = table.to(self.rt.device)
         self.table = self.rt.shared[key]
 

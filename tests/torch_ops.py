@@ -200,7 +200,7 @@ class TorchOps:
             return self._gn(also_norm.to(torch.float32), also_weight, 1, eps).to(x.dtype)
         return None
 
-    def head_linear(self, x, x_head, weight, out, out_head, gate=None, rope_tail=None):
+    def head_linear(self, x, x_head, weight, out, out_head, gate=None, rope_tail=None, gate_wide=False):
         H, O, K = weight.shape
         if rope_tail is not None:
             x_at, out_at, width, positions, table = rope_tail
@@ -208,7 +208,8 @@ class TorchOps:
         for h in range(H):
             y = x[:, h * x_head:h * x_head + K].to(torch.float32) @ weight[h].to(torch.float32).t()
             if gate is not None:
-                y = y * torch.sigmoid(gate[:, h:h + 1].to(torch.float32))
+                g = gate[:, h * O:(h + 1) * O] if gate_wide else gate[:, h:h + 1]
+                y = y * torch.sigmoid(g.to(torch.float32))
             out[:, h * out_head:h * out_head + O] = y.to(out.dtype)
         return out
 
@@ -219,18 +220,68 @@ class TorchOps:
             out[:, h * out_head + out_at:h * out_head + out_at + width] = self._rotate(v, cs, table.shape[1]).to(out.dtype)
             out[:, h * out_head + out_at + width:(h + 1) * out_head] = 0
 
-    def table_moe(self, h, w_gate_up, w_down, token_ids, table, weight, base=None):
+    def table_moe(self, h, w_gate_up, w_down, token_ids, table, weight, base=None, pair_scale=None, base_scale=None):
         F = w_gate_up.shape[1] // 2
         out = torch.zeros(h.shape, dtype=torch.float32)
         for n in range(h.shape[0]):
-            for e in table[int(token_ids[n])].tolist():
-                gu = (w_gate_up[e].to(torch.float32) @ h[n].to(torch.float32)).to(h.dtype).to(torch.float32)
+            for k, e in enumerate(table[int(token_ids[n]) if token_ids is not None else n].tolist()):
+                x = h[n].to(torch.float32) * (float(pair_scale[n, k]) if pair_scale is not None else 1.0)
+                gu = (w_gate_up[e].to(torch.float32) @ x).to(h.dtype).to(torch.float32)
                 a = (gu[:F] / (1.0 + torch.exp(-gu[:F])) * gu[F:]).to(h.dtype).to(torch.float32)
                 out[n] += w_down[e].to(torch.float32) @ a
         out = out * weight
         if base is not None:
-            out = out + base.to(torch.float32)
+            b = base.to(torch.float32)
+            out = out + (b * base_scale[:, None] if base_scale is not None else b)
         return out.to(h.dtype)
+
+    def moe_route(self, logits, experts, top, renorm=False, extra=-1):
+        s = torch.sigmoid(logits[:, :experts])
+        # the largest first, the lower index among equals
+        order = torch.argsort(-logits[:, :experts], dim=-1, stable=True)[:, :top]
+        w = torch.gather(s, 1, order)
+        if renorm:
+            w = w / w.sum(-1, keepdim=True)
+        gate = torch.sigmoid(logits[:, extra]).contiguous() if extra >= 0 else None
+        return order.to(torch.int32).contiguous(), w.contiguous(), gate
+
+    def scale_add_norm(self, a, scale_a, b, scale_b, residual, weight=None, eps=1e-5):
+        r = residual + scale_a * a.to(torch.float32)
+        if b is not None:
+            r = r + scale_b * b.to(torch.float32)
+        residual.copy_(r)
+        if weight is None:
+            return None
+        return (r / torch.sqrt((r * r).mean(-1, keepdim=True) + eps) * weight.to(torch.float32)).to(a.dtype)
+
+    def logit_cap(self, logits, scale=1.0, cap=0.0):
+        y = logits * scale
+        logits.copy_(cap * torch.tanh(y / cap) if cap > 0 else y)
+        return logits
+
+    def retention_state_floats(self, heads, dim, vdim):
+        return heads * dim * vdim
+
+    def retention(self, q, k, v, decay, out_gate, state, batch, heads, dim, vdim, q_scale, eps, table=None):
+        H, d, dv = heads, dim, vdim
+        out = torch.empty((q.shape[0], H * dv), dtype=q.dtype)
+        g = decay[:H]
+        for a, b, slot in self._segments(batch):
+            S = state[slot, :H * d * dv].reshape(H, d, dv).clone()
+            for t in range(a, b):
+                qt = q[t, :H * d].to(torch.float32).reshape(H, d)
+                kt = k[t, :H * d].to(torch.float32).reshape(H, d)
+                if table is not None:
+                    cs = table[int(batch.positions[t])]
+                    qt, kt = self._rotate(qt, cs, table.shape[1]), self._rotate(kt, cs, table.shape[1])
+                vt = v[t, :H * dv].to(torch.float32).reshape(H, dv)
+                S = g[:, None, None] * S + kt[:, :, None] * vt[:, None, :]
+                o = torch.einsum("hdv,hd->hv", S, qt * q_scale)
+                o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps)
+                gt = out_gate[t, :H * dv].to(torch.float32)
+                out[t] = (o.reshape(-1) * (gt / (1.0 + torch.exp(-gt)))).to(q.dtype)
+            state[slot, :H * d * dv] = S.reshape(-1)
+        return out
 
     # ------------------------------------------------------------ Dynamic Tanh, state-carrying mixers
     def dyt_norm(self, branch, residual, weight, bias, alpha, out_dtype, rows=None):
