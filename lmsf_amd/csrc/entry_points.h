@@ -204,12 +204,12 @@ long lmsf_retention_chunk_entry_floats(int H, int d, int dv);
 int lmsf_retention_chunked(const void* q, const void* k, const void* v, int dtype, long qkv_stride,
     const int* positions, const float* table, int rot, int max_pos, const float* decay, const void* og,
     long og_stride, float* state, long state_stride, const int* seg_starts, const int* state_slots, void* out,
-    long out_stride, float* o_raw, int n_tokens, int n_segments, int H, int d, int dv, float qscale, float eps,
+    long out_stride, float* o_raw, int n_tokens, int n_segments, int H, int d, int dv, float kscale, float eps,
     const int* chunk_base, int max_chunks, long n_entries, float* entries, hipStream_t stream);
 int lmsf_retention_tokens(const void* q, const void* k, const void* v, int dtype, long qkv_stride,
     const int* positions, const float* table, int rot, int max_pos, const float* decay, const void* og,
     long og_stride, float* state, long state_stride, const int* seg_starts, const int* state_slots, void* out,
-    long out_stride, float* o_raw, int n_tokens, int n_segments, int H, int d, int dv, float qscale, float eps,
+    long out_stride, float* o_raw, int n_tokens, int n_segments, int H, int d, int dv, float kscale, float eps,
     hipStream_t stream);
 
 // layer_scale.hip

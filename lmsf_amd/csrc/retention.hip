@@ -1,8 +1,8 @@
 // Retention: linear attention with a fixed decay per head and no softmax or denominator. Per head, with decay g:
 //   S_t = g S_(t-1) + k_t v_t^T,   o_t = S_t^T q_t,   out_t = o_t / rms(o_t) * silu(gate_t)
 // (rms over the head's dv entries, eps inside the root, no weight). q and k are rotated by the token's position
-// (pairs (i, i + rot/2) of the first ``rot`` entries, cos and sin from a float32 table) on their way in; q is
-// multiplied by ``qscale`` (a factor on k is a factor on q: o is linear in both). The state of a slot is S as
+// (pairs (i, i + rot/2) of the first ``rot`` entries, cos and sin from a float32 table) on their way in; k is then
+// multiplied by ``kscale``. The state of a slot is S as
 // [H, d, dv] float32, all zeros when a request begins. The reference has no such mixer (its only one is attention
 // over a paged cache, core/src/model_executor/layers/attention.rs:91-231).
 //
@@ -48,7 +48,7 @@ __global__ __launch_bounds__(RET_THREADS) void retention_chunk_kernel(
     const int* __restrict__ positions, const float* __restrict__ table, int rot, int max_pos,
     const float* __restrict__ log_decay, float* __restrict__ state, long state_stride,
     const int* __restrict__ seg_starts, const int* __restrict__ state_slots, float* __restrict__ o_raw, long o_stride,
-    int H, int d, int dv, int L, float qscale, int n_vb, const int* __restrict__ chunk_base, float* __restrict__ sc_U) {
+    int H, int d, int dv, int L, float kscale, int n_vb, const int* __restrict__ chunk_base, float* __restrict__ sc_U) {
   extern __shared__ float lds[];
   const int dp = d | 1, NCp = RET_DVB | 1, Lp = L | 1;
   float* sq = lds;                  // [L][dp]
@@ -79,8 +79,8 @@ __global__ __launch_bounds__(RET_THREADS) void retention_chunk_kernel(
       const int tt = i / d, dd = i % d;
       const long row = (long)(t0 + tt) * qkv_stride + (long)h * d;
       const float* cs = table ? table + (long)min(max(positions[t0 + tt], 0), max_pos - 1) * rot : nullptr;
-      if (MODE != 1) sq[tt * dp + dd] = (cs ? ret_rotated<T>(q + row, cs, dd, rot) : to_f32<T>(q[row + dd])) * qscale;
-      sk[tt * dp + dd] = cs ? ret_rotated<T>(k + row, cs, dd, rot) : to_f32<T>(k[row + dd]);
+      if (MODE != 1) sq[tt * dp + dd] = cs ? ret_rotated<T>(q + row, cs, dd, rot) : to_f32<T>(q[row + dd]);
+      sk[tt * dp + dd] = (cs ? ret_rotated<T>(k + row, cs, dd, rot) : to_f32<T>(k[row + dd])) * kscale;
     }
     for (int i = tid; i < nt * nb; i += RET_THREADS) {
       const int tt = i / nb, c = i % nb;
@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) void retention_token_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, long qkv_stride,
     const int* __restrict__ positions, const float* __restrict__ table, int rot, int max_pos,
     const float* __restrict__ decay, float* __restrict__ state, long state_stride, const int* __restrict__ seg_starts,
-    const int* __restrict__ state_slots, float* __restrict__ o_raw, long o_stride, int H, int d, int dv, float qscale) {
+    const int* __restrict__ state_slots, float* __restrict__ o_raw, long o_stride, int H, int d, int dv, float kscale) {
   extern __shared__ float lds[];
   float* sq = lds;               // [d]
   float* sk = sq + d;            // [d]
@@ -213,8 +213,8 @@ __global__ __launch_bounds__(256) void retention_token_kernel(
     const long row = (long)t * qkv_stride + (long)h * d;
     const float* cs = table ? table + (long)min(max(positions[t], 0), max_pos - 1) * rot : nullptr;
     for (int i = tid; i < d; i += 256) {
-      sq[i] = (cs ? ret_rotated<T>(q + row, cs, i, rot) : to_f32<T>(q[row + i])) * qscale;
-      sk[i] = cs ? ret_rotated<T>(k + row, cs, i, rot) : to_f32<T>(k[row + i]);
+      sq[i] = cs ? ret_rotated<T>(q + row, cs, i, rot) : to_f32<T>(q[row + i]);
+      sk[i] = (cs ? ret_rotated<T>(k + row, cs, i, rot) : to_f32<T>(k[row + i])) * kscale;
     }
     const float vv = col_ok ? to_f32<T>(v[(long)t * qkv_stride + (long)h * dv + e0 + lane]) : 0.f;
     __syncthreads();
@@ -292,7 +292,7 @@ extern "C" int lmsf_retention_chunked(const void* q, const void* k, const void* 
                                       const float* decay, const void* og, long og_stride, float* state,
                                       long state_stride, const int* seg_starts, const int* state_slots, void* out,
                                       long out_stride, float* o_raw, int n_tokens, int n_segments, int H, int d, int dv,
-                                      float qscale, float eps, const int* chunk_base, int max_chunks, long n_entries,
+                                      float kscale, float eps, const int* chunk_base, int max_chunks, long n_entries,
                                       float* entries, hipStream_t stream) {
   if (ret_check(q, k, v, dtype, qkv_stride, positions, table, rot, max_pos, decay, og, og_stride, state, state_stride,
                 seg_starts, state_slots, out, out_stride, o_raw, n_tokens, n_segments, H, d, dv))
@@ -319,7 +319,7 @@ extern "C" int lmsf_retention_chunked(const void* q, const void* k, const void* 
     }                                                                                                                \
     hipLaunchKernelGGL((retention_chunk_kernel<T, MODE>), GRID, dim3(RET_THREADS), smem, stream, (const T*)q,        \
                        (const T*)k, (const T*)v, qkv_stride, positions, table, rot, max_pos, log_decay, state,       \
-                       state_stride, seg_starts, state_slots, o_raw, (long)H * dv, H, d, dv, L, qscale, n_vb,        \
+                       state_stride, seg_starts, state_slots, o_raw, (long)H * dv, H, d, dv, L, kscale, n_vb,        \
                        chunk_base, entries);                                                                         \
   } while (0)
   if (!chunk_base) {
@@ -350,7 +350,7 @@ extern "C" int lmsf_retention_tokens(const void* q, const void* k, const void* v
                                      const float* decay, const void* og, long og_stride, float* state,
                                      long state_stride, const int* seg_starts, const int* state_slots, void* out,
                                      long out_stride, float* o_raw, int n_tokens, int n_segments, int H, int d, int dv,
-                                     float qscale, float eps, hipStream_t stream) {
+                                     float kscale, float eps, hipStream_t stream) {
   if (ret_check(q, k, v, dtype, qkv_stride, positions, table, rot, max_pos, decay, og, og_stride, state, state_stride,
                 seg_starts, state_slots, out, out_stride, o_raw, n_tokens, n_segments, H, d, dv))
     return 1;
@@ -361,13 +361,13 @@ extern "C" int lmsf_retention_tokens(const void* q, const void* k, const void* v
   if (dtype == LMSF_F32) {
     hipLaunchKernelGGL((retention_token_kernel<float>), grid, block, smem, stream, (const float*)q, (const float*)k,
                        (const float*)v, qkv_stride, positions, table, rot, max_pos, decay, state, state_stride,
-                       seg_starts, state_slots, o_raw, (long)H * dv, H, d, dv, qscale);
+                       seg_starts, state_slots, o_raw, (long)H * dv, H, d, dv, kscale);
     LMSF_LAUNCH_CHECK("retention_tokens");
     ret_heads<float>(o_raw, og, og_stride, out, out_stride, n_tokens, H, dv, eps, stream);
   } else {
     hipLaunchKernelGGL((retention_token_kernel<bf16_t>), grid, block, smem, stream, (const bf16_t*)q, (const bf16_t*)k,
                        (const bf16_t*)v, qkv_stride, positions, table, rot, max_pos, decay, state, state_stride,
-                       seg_starts, state_slots, o_raw, (long)H * dv, H, d, dv, qscale);
+                       seg_starts, state_slots, o_raw, (long)H * dv, H, d, dv, kscale);
     LMSF_LAUNCH_CHECK("retention_tokens");
     ret_heads<bf16_t>(o_raw, og, og_stride, out, out_stride, n_tokens, H, dv, eps, stream);
   }

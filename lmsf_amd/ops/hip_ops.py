@@ -831,10 +831,10 @@ class HipOps:
         return int(self.lib.lmsf_retention_state_floats(heads, dim, vdim))
 
     def retention(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor, out_gate: torch.Tensor,
-                  state: torch.Tensor, batch, heads: int, dim: int, vdim: int, q_scale: float, eps: float,
+                  state: torch.Tensor, batch, heads: int, dim: int, vdim: int, k_scale: float, eps: float,
                   table: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Linear attention with a fixed decay per head over each request's tokens, the memory S [heads, dim, vdim]
-        carried in ``state`` (float32 [slots, >= heads * dim * vdim]): S <- decay S + k v^T, o = S^T (q * q_scale);
+        carried in ``state`` (float32 [slots, >= heads * dim * vdim]): S <- decay S + (k * k_scale) v^T, o = S^T q;
         returns every head's o over its root mean square times silu(out_gate), [N, heads * vdim] in q's dtype.
         q, k [N, heads * dim] and v [N, heads * vdim]: views of one buffer (equal row strides). ``decay``: float32
         [2 heads], the decays and then their logarithms. ``table`` (float32 [max_pos, rot] = [cos | sin]): q and k
@@ -863,7 +863,7 @@ class HipOps:
         head = (_ptr(q), _ptr(k), _ptr(v), _code(q.dtype), q.stride(0), _ptr(batch.positions) if table is not None else None,
                 _ptr(table), rot, max_pos, _ptr(decay), _ptr(out_gate), out_gate.stride(0), _ptr(state), state.stride(0),
                 _ptr(seg_starts), _ptr(slots), _ptr(out), out.stride(0), _ptr(raw), N, S, int(heads), int(dim), int(vdim),
-                float(q_scale), float(eps))
+                float(k_scale), float(eps))
         lens = getattr(batch, "host_seg_lens", None)
         L = self.lib.lmsf_retention_chunk_tokens(int(dim))
         if not getattr(batch, "replayed", False) and not getattr(batch, "all_single", False) and lens and L > 0 \

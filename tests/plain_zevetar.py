@@ -149,8 +149,10 @@ def routed_experts(h, mlp, t, pre, storage):
     score times h as input; the shared expert's result times sigmoid(w_sg . h)."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
     hs = _rt(h, storage)
-    s = torch.sigmoid(hs @ t[pre + "router"].T)
-    w, idx = torch.topk(s, top, dim=-1)
+    z = hs @ t[pre + "router"].T
+    # (the largest scores are the largest logits; chosen by the logits, two scores that both round to 1 stay apart)
+    idx = torch.topk(z, top, dim=-1).indices
+    w = torch.sigmoid(torch.gather(z, 1, idx))
     out = torch.zeros_like(h)
     for e in range(E):
         for kk in range(top):

@@ -262,7 +262,7 @@ class TorchOps:
     def retention_state_floats(self, heads, dim, vdim):
         return heads * dim * vdim
 
-    def retention(self, q, k, v, decay, out_gate, state, batch, heads, dim, vdim, q_scale, eps, table=None):
+    def retention(self, q, k, v, decay, out_gate, state, batch, heads, dim, vdim, k_scale, eps, table=None):
         H, d, dv = heads, dim, vdim
         out = torch.empty((q.shape[0], H * dv), dtype=q.dtype)
         g = decay[:H]
@@ -275,8 +275,8 @@ class TorchOps:
                     cs = table[int(batch.positions[t])]
                     qt, kt = self._rotate(qt, cs, table.shape[1]), self._rotate(kt, cs, table.shape[1])
                 vt = v[t, :H * dv].to(torch.float32).reshape(H, dv)
-                S = g[:, None, None] * S + kt[:, :, None] * vt[:, None, :]
-                o = torch.einsum("hdv,hd->hv", S, qt * q_scale)
+                S = g[:, None, None] * S + (kt * k_scale)[:, :, None] * vt[:, None, :]
+                o = torch.einsum("hdv,hd->hv", S, qt)
                 o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps)
                 gt = out_gate[t, :H * dv].to(torch.float32)
                 out[t] = (o.reshape(-1) * (gt / (1.0 + torch.exp(-gt)))).to(q.dtype)
