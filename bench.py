@@ -461,6 +461,34 @@ def niresun_shapes(name):
     return nire, llama
 
 
+def zevetar_shapes(name):
+    """A Zevetar configuration at sizes that resemble a real model's layers, and beside it the Takosun configuration
+    of equal width, depth, feed-forward sizes and latent attention (the closest architecture of the package: latent
+    attention, routed experts with a shared one). Zevetar's layers go round latent attention with a window and a dense
+    feed-forward, latent attention on the same latent with experts, retention with experts, retention with a dense
+    feed-forward; every layer runs its mixer and its feed-forward side by side on one norm."""
+    tako, _ = takosun_shapes(name)
+    # retention: heads, key size, value size; the window of the attention layers
+    RH, rd, rdv, window = {"2b": (16, 64, 128, 1024), "7b": (32, 64, 128, 1024)}[name]
+    first, second = tako["layers"][0], tako["layers"][1]
+    layers = []
+    for i in range(len(tako["layers"])):
+        if i % 4 < 2:
+            m = dict((first, second)[i % 2]["mixer"], mask={"size": window})
+            m["rot"] = dict(m["rot"], scaling={"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0})
+            if i % 2:
+                m["kv_from"] = i - 1
+            layers.append({"type": "latent_attention", "mixer": m, "mlp": (first, second)[i % 2]["mlp"]})
+        else:
+            m = {"heads": RH, "dim": rd, "vdim": rdv, "decay": [1.0 - 2.0 ** (-5 - 7.0 * h / RH) for h in range(RH)],
+                 "rot": {"base": 1e6, "dims": rd}}
+            layers.append({"type": "retention", "mixer": m, "mlp": (second, first)[i % 2]["mlp"]})
+    zev = {"architecture": "Zevetar", "vocab": tako["vocab"], "width": tako["width"], "norm": {"eps": 1e-6},
+           "embedding": {"scale": tako["width"] ** 0.5}, "logit_scale": 0.5, "logit_softcap": 30.0, "layers": layers,
+           "max_position_embeddings": 8192, "torch_dtype": "bfloat16"}
+    return zev, tako
+
+
 def takosun_run(args):
     """``--workload takosun``: prefill and decode of a Takosun model beside the Llama model of equal size; one JSON
     line. Decode: ``--steps`` steps at batch 1, 8 and 64 after 512-token prompts; prefill: one request of 512 and of
@@ -473,12 +501,17 @@ def niresun_run(args):
     beside_llama_run(args, "niresun", args.niresun_sizes, niresun_shapes(args.niresun_sizes))
 
 
-def beside_llama_run(args, design, sizes, shapes):
+def zevetar_run(args):
+    """``--workload zevetar``: the same for a Zevetar model, beside the Takosun model of equal size."""
+    beside_llama_run(args, "zevetar", args.zevetar_sizes, zevetar_shapes(args.zevetar_sizes), twin="takosun")
+
+
+def beside_llama_run(args, design, sizes, shapes, twin="llama"):
     import gc
     import torch
-    out = {"metric": "%s_beside_llama" % design, "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
+    out = {"metric": "%s_beside_%s" % (design, twin), "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
            "steps": args.steps, "warmup": args.warmup, "config": {"sizes": sizes}, "models": {}}
-    for name, cfg in zip((design, "llama"), shapes):
+    for name, cfg in zip((design, twin), shapes):
         engine = make_engine(cfg, args, max_num_seqs=64, dtype=args.dtype)
         m = {"weight_gb": round(weight_bytes(engine) / 1e9, 3),
              "decode_graphs": bool(engine.core.executor.use_graphs), "step_program": engine.core.executor.program is not None}
@@ -494,8 +527,8 @@ def beside_llama_run(args, design, sizes, shapes):
         del engine
         gc.collect()
         torch.cuda.empty_cache()
-    t, l = out["models"][design], out["models"]["llama"]
-    out["%s_over_llama" % design] = {k: round(t[k] / l[k], 3) for k in t if k.endswith("tok_s")}
+    t, l = out["models"][design], out["models"][twin]
+    out["%s_over_%s" % (design, twin)] = {k: round(t[k] / l[k], 3) for k in t if k.endswith("tok_s")}
     out["value"], out["higher_is_better"] = t["decode_b8_tok_s"], True
     print(json.dumps(out))
 
@@ -523,14 +556,17 @@ def main():
     ap.add_argument("--max-num-batched-tokens", type=int, default=8192)
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.85)
     ap.add_argument("--skip-points", action="store_true", help="leave out the batch 1 and batch 64 runs")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "products", "takosun", "niresun"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "products", "takosun", "niresun", "zevetar"],
                     help="decode: the default line (Llama-3-8B shape); serve: continuous batching of 64 requests at "
                          "Llama-2-7B shape, a line of its own; products: a layer's matrix products alone, the "
                          "library's against the engine's choice, at --rows; takosun: a Takosun model beside the Llama model "
-                         "of equal size, prefill and decode")
+                         "of equal size, prefill and decode; niresun: the same for a Niresun model; zevetar: a Zevetar "
+                         "model beside the Takosun model of equal size")
     ap.add_argument("--takosun-sizes", default="2b", choices=["2b", "7b"], help="takosun: the layers' sizes")
     ap.add_argument("--niresun-sizes", default="2b", choices=["2b", "7b"],
                     help="niresun: the layers' sizes (a Niresun model beside the Llama model of equal size)")
+    ap.add_argument("--zevetar-sizes", default="2b", choices=["2b", "7b"],
+                    help="zevetar: the layers' sizes (a Zevetar model beside the Takosun model of equal size)")
     ap.add_argument("--rows", default="17,64,100,128,129,192,256,512,2048", help="products: numbers of rows")
     ap.add_argument("--prefill-chunk-size", type=int, default=1024, help="serve: longest portion of a prompt in a step")
     ap.add_argument("--shape", default="llama3-8b", choices=sorted(SHAPES),
@@ -571,6 +607,9 @@ def main():
         return
     if args.workload == "niresun":
         niresun_run(args)
+        return
+    if args.workload == "zevetar":
+        zevetar_run(args)
         return
     import torch
     shape_name, shape_cfg = SHAPES[args.shape]

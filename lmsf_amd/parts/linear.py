@@ -19,12 +19,14 @@ class FusedLinear(Part):
     shape [rows, in_features] and, with ``bias``, ``prefix.sub-name.bias`` has [rows]. With ``bare_names`` the
     matrix is the tensor ``prefix.sub-name`` itself (checkpoints that name a matrix without ".weight").
     ``bias`` may also list the sub-names that have a bias (the others' rows of the fused bias are zeros);
-    ``bias_name`` is what a bias is called after its matrix's name ("bias", or "b")."""
+    ``bias_name`` is what a bias is called after its matrix's name ("bias", or "b"). ``pad_rows_to``: rows of zeros
+    follow the sources' so that the fused matrix has a multiple of that many (a kernel that wants its outputs in
+    eights; the result then has as many columns more, all zeros)."""
 
     graph_safe = True
 
     def __init__(self, prefix: str, rt: Runtime, in_features: int, sources: Sequence[Tuple[str, int]],
-                 bias=False, bare_names: bool = False, bias_name: str = "bias", row_orders=None):
+                 bias=False, bare_names: bool = False, bias_name: str = "bias", row_orders=None, pad_rows_to: int = 1):
         super().__init__(prefix, rt)
         # sub-name -> for every row of the loaded source the checkpoint row it holds (a mixer that wants its
         # outputs in another order than the checkpoint's, e.g. rotation pairs side by side instead of interleaved)
@@ -37,6 +39,9 @@ class FusedLinear(Part):
         self.in_features = int(in_features)
         self.sources = [(str(n), int(r)) for n, r in sources]
         self.out_features = sum(r for _, r in self.sources)
+        if int(pad_rows_to) < 1:
+            raise ValueError("FusedLinear: pad_rows_to must be >= 1")
+        self.rows_held = -(-self.out_features // int(pad_rows_to)) * int(pad_rows_to)
         self.has_bias = bool(bias) if isinstance(bias, bool) else bool(self.biased)
         self.weight: Optional[torch.Tensor] = None
         self.bias: Optional[torch.Tensor] = None
@@ -64,10 +69,10 @@ class FusedLinear(Part):
         kernels ask for (``ops.weight_row_pad``: a few elements more than a row holds, so that rows do not all
         begin on the same memory channel); what is returned is the [out, in] view of it."""
         if what != "weight":
-            return torch.empty((self.out_features,), dtype=dtype, device=device)
+            return torch.empty((self.rows_held,), dtype=dtype, device=device)
         pad_of = getattr(self.rt.ops, "weight_row_pad", None)
         pad = int(pad_of(self.in_features, dtype)) if pad_of is not None else 0
-        buf = torch.empty((self.out_features, self.in_features + pad), dtype=dtype, device=device)
+        buf = torch.empty((self.rows_held, self.in_features + pad), dtype=dtype, device=device)
         return buf[:, :self.in_features]
 
     def _gather(self, fetch: Callable[[str], torch.Tensor], what: str) -> torch.Tensor:
@@ -95,6 +100,8 @@ class FusedLinear(Part):
             out[row:row + rows].copy_(t)
             row += rows
             del t
+        if row < self.rows_held:
+            out[row:].zero_()
         return out
 
     def load_weights(self, fetch: Callable[[str], torch.Tensor]) -> None:

@@ -41,8 +41,9 @@ class RoutedMoE(FeedForward):
             raise ValueError("%s: a gate without a shared expert" % prefix)
         sources = [(router_name, self.E)] + ([(shared_gate, 1)] if shared_gate is not None else [])
         self.has_shared_gate = shared_gate is not None
-        # the router (and the shared expert's gate) as one product with a float32 result
-        self.router = FusedLinear(prefix, rt, self.W, sources, bare_names=True)
+        # the router (and the shared expert's gate) as one product with a float32 result; rows of zeros make them a
+        # multiple of eight, which the many-rows form of that product asks for
+        self.router = FusedLinear(prefix, rt, self.W, sources, bare_names=True, pad_rows_to=8)
         self.w_gate_up: Optional[torch.Tensor] = None     # [E, 2F, W]
         self.w_down: Optional[torch.Tensor] = None        # [E, W, F]
 
@@ -71,7 +72,7 @@ class RoutedMoE(FeedForward):
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         ops = self.rt.ops
-        logits = ops.linear_wide(h, self.router.weight, None)                       # float32 [N, E (+ 1)]
+        logits = ops.linear_wide(h, self.router.weight, None)                       # float32 [N, >= E (+ 1)]
         choice, weight, gate = ops.moe_route(logits, self.E, self.top, renorm=self.renormalize,
                                              extra=self.E if self.has_shared_gate else -1)
         base = self.shared.forward(h) if self.shared is not None else None

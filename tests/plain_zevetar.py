@@ -1,8 +1,8 @@
 """A plain, slow implementation of the Zevetar design: whole sequences, no cache, recurrences token by token, one
 function per mechanism. It shares nothing with the package: it reads a configuration dictionary and a dictionary of
 tensors by checkpoint name. ``dtype`` float64 gives the yardstick, float32 what float32 rounding costs; ``storage``
-(a torch dtype or None) rounds what an engine may keep in 16 bits: the operands and results of the projections and
-the activations between them.
+(a torch dtype, None, or a pair (dtype, generator) for another draw of the rounding errors) rounds what an engine may
+keep in 16 bits: the operands and results of the projections and the activations between them.
 
 Notation: T tokens, width W. A layer is x += ls1 * mixer(h) + ls2 * ffn(h) with h = rms_norm(x; w1): one norm, both
 sublayers read it, each result is scaled entry by entry before the sum.
@@ -13,8 +13,15 @@ import torch
 
 
 def _rt(x, storage):
-    """Round to the storage type and back (what a 16-bit buffer does to a value)."""
-    return x if storage is None else x.to(storage).to(x.dtype)
+    """Round to the storage type and back (what a 16-bit buffer does to a value). ``storage`` may be (type, generator):
+    the value is then moved by up to half a bfloat16 step at random before it is rounded, which gives another draw
+    of the rounding errors (an engine that adds up in another order rounds some values the other way)."""
+    if storage is None:
+        return x
+    if isinstance(storage, tuple):
+        storage, gen = storage
+        x = x * (1.0 + (torch.rand(x.shape, generator=gen, dtype=torch.float32).to(x.dtype) - 0.5) * 2.0 ** -8)
+    return x.to(storage).to(x.dtype)
 
 
 def rms_norm(x, w, eps):
