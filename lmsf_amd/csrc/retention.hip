@@ -10,7 +10,9 @@
 // after the other in a workgroup; chunks side by side (summaries, a fold, outputs) for long segments; and token by
 // token with the state streamed once for steps of single tokens. Over a chunk with first state S_0:
 //   P[t][u] = (q_t . k_u) g^(t-u) for u <= t;   O = diag(g^(t+1)) Q S_0 + P V;   S_L = g^L S_0 + K^T diag(g^(L-1-u)) V.
-// Powers of g are exp(n log g) in float32. Everything is float32 but the operands as they are stored.
+// Powers of g are exp(n log g) in float32. Everything is float32 but the operands as they are stored. The chunked
+// forms run their products on the matrix cores in float32 where a head's operands fit LDS (heads of up to 256
+// entries), with scalar multiply-adds otherwise.
 #include "common.h"
 #include "entry_points.h"
 
@@ -141,6 +143,168 @@ __global__ __launch_bounds__(RET_THREADS) void retention_chunk_kernel(
   }
 }
 
+// The same three forms with the products on the matrix cores in float32 (v_mfma_f32_16x16x4_f32: full float32
+// operands and sums). A workgroup of sixteen waves takes a head, a chunk and RM_NB value columns; every size is padded
+// with zeros to a multiple of 16 in LDS. A wave computes tiles of 16 x 16: of P = Q K^T (at and below the diagonal,
+// masked and decayed as it is stored), of O = diag(g^(t+1)) Q S_0 + P V (the second product as far as the diagonal)
+// and of S_L = g^L S_0 + K^T (w V). Rows of operands whose row is the product's inner index lie RM_BS apart, the
+// others a multiple of 16 plus 4, so that a wave's 64 operand reads fall into 64 banks.
+#define RM_THREADS 1024
+#define RM_NB 64
+#define RM_BS (RM_NB + 16)
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(RM_THREADS) void retention_chunk_mfma_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, long qkv_stride,
+    const int* __restrict__ positions, const float* __restrict__ table, int rot, int max_pos,
+    const float* __restrict__ log_decay, float* __restrict__ state, long state_stride,
+    const int* __restrict__ seg_starts, const int* __restrict__ state_slots, float* __restrict__ o_raw, long o_stride,
+    int H, int d, int dv, int L, float kscale, int n_vb, const int* __restrict__ chunk_base, float* __restrict__ sc_U) {
+  extern __shared__ float lds[];
+  const int d16 = (d + 15) / 16 * 16, dq = d16 + 4, Lq = L + 4;
+  float* sq = lds;                  // [L][dq]
+  float* sk = sq + L * dq;          // [L][dq]
+  float* sv = sk + L * dq;          // [L][RM_BS]
+  float* sP = sv + L * RM_BS;       // [L][Lq]
+  float* sS = sP + L * Lq;          // [d16][RM_BS]
+  float* sw = sS + d16 * RM_BS;     // [L]
+  const int tid = threadIdx.x, wave = tid / LMSF_WAVE, lane = tid % LMSF_WAVE, fr = lane % 16, fg = lane / 16;
+  const int h = blockIdx.x, s = blockIdx.y;
+  const int vb = MODE == 0 ? blockIdx.z : blockIdx.z % n_vb, j = MODE == 0 ? 0 : blockIdx.z / n_vb;
+  const int e0 = vb * RM_NB, nb = min(RM_NB, dv - e0);
+  const int seg_start = seg_starts[s], seg_end = seg_starts[s + 1];
+  if (MODE != 0 && j * L >= seg_end - seg_start) return;
+  const int start = MODE == 0 ? seg_start : seg_start + j * L;
+  const int end = MODE == 0 ? seg_end : min(seg_end, start + L);
+  const float lg = log_decay[h];
+  const int nRT = L / 16, nCT = (nb + 15) / 16, nDT = d16 / 16;
+  float* gS = MODE == 0 ? state + (long)state_slots[s] * state_stride + (long)h * d * dv
+                        : sc_U + (((long)chunk_base[s] + j) * H + h) * d * dv;
+  if (MODE != 1)
+    for (int i = tid; i < d16 * RM_NB; i += RM_THREADS) {
+      const int dd = i / RM_NB, c = i % RM_NB;
+      sS[dd * RM_BS + c] = dd < d && c < nb ? gS[(long)dd * dv + e0 + c] : 0.f;
+    }
+  for (int t0 = start; t0 < end; t0 += L) {
+    const int nt = min(L, end - t0);
+    __syncthreads();
+    // a row's units: the rotated pairs (e, e + half), then the entries that pass unchanged and the padding
+    const int rotn = table ? rot : 0, half = rotn / 2, per_row = half + (d16 - rotn);
+#pragma unroll 2
+    for (int i = tid; i < L * per_row; i += RM_THREADS) {
+      const int tt = i / per_row, e = i % per_row;
+      const bool live = tt < nt;
+      const long row = (long)(t0 + min(tt, nt - 1)) * qkv_stride + (long)h * d;
+      if (e < half) {
+        float qa = 0.f, qb = 0.f, ka = 0.f, kb = 0.f;
+        if (live) {
+          const float* cs = table + (long)min(max(positions[t0 + tt], 0), max_pos - 1) * rot;
+          const float c = cs[e], sn = cs[half + e];
+          if (MODE != 1) rope_rotate(to_f32<T>(q[row + e]), to_f32<T>(q[row + e + half]), c, sn, &qa, &qb);
+          rope_rotate(to_f32<T>(k[row + e]), to_f32<T>(k[row + e + half]), c, sn, &ka, &kb);
+        }
+        if (MODE != 1) sq[tt * dq + e] = qa, sq[tt * dq + e + half] = qb;
+        sk[tt * dq + e] = ka * kscale, sk[tt * dq + e + half] = kb * kscale;
+      } else {
+        const int dd = rotn + e - half;
+        const bool in = live && dd < d;
+        if (MODE != 1) sq[tt * dq + dd] = in ? to_f32<T>(q[row + dd]) : 0.f;
+        sk[tt * dq + dd] = in ? to_f32<T>(k[row + dd]) * kscale : 0.f;
+      }
+    }
+#pragma unroll 4
+    for (int i = tid; i < L * RM_NB; i += RM_THREADS) {
+      const int tt = i / RM_NB, c = i % RM_NB;
+      sv[tt * RM_BS + c] =
+          tt < nt && c < nb ? to_f32<T>(v[(long)(t0 + tt) * qkv_stride + (long)h * dv + e0 + c]) : 0.f;
+    }
+    if (MODE != 2)
+      for (int i = tid; i < L; i += RM_THREADS) sw[i] = i < nt ? ret_pow(lg, nt - 1 - i) : 0.f;
+    __syncthreads();
+    if (MODE != 1) {
+      for (int tile = wave; tile < nRT * nRT; tile += RM_THREADS / LMSF_WAVE) {
+        const int rt = tile / nRT, ct = tile % nRT;
+        if (ct > rt) continue;
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+        const float* ap = sq + (rt * 16 + fr) * dq + fg;
+        const float* bp = sk + (ct * 16 + fr) * dq + fg;
+#pragma unroll 4
+        for (int kk = 0; kk < d16; kk += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ap[kk], bp[kk], acc, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int t = rt * 16 + fg * 4 + r, u = ct * 16 + fr;
+          sP[t * Lq + u] = u <= t ? acc[r] * ret_pow(lg, t - u) : 0.f;
+        }
+      }
+      __syncthreads();
+      for (int tile = wave; tile < nRT * nCT; tile += RM_THREADS / LMSF_WAVE) {
+        const int rt = tile / nCT, ct = tile % nCT;
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+        const float* ap = sq + (rt * 16 + fr) * dq + fg;
+        const float* bp = sS + fg * RM_BS + ct * 16 + fr;
+#pragma unroll 4
+        for (int kk = 0; kk < d16; kk += 4)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ap[kk], bp[kk * RM_BS], acc, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[r] *= ret_pow(lg, rt * 16 + fg * 4 + r + 1);
+        ap = sP + (rt * 16 + fr) * Lq + fg;
+        bp = sv + fg * RM_BS + ct * 16 + fr;
+#pragma unroll 4
+        for (int kk = 0; kk < (rt + 1) * 16; kk += 4)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ap[kk], bp[kk * RM_BS], acc, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int t = rt * 16 + fg * 4 + r, c = ct * 16 + fr;
+          if (t < nt && c < nb) o_raw[(long)(t0 + t) * o_stride + (long)h * dv + e0 + c] = acc[r];
+        }
+      }
+    }
+    if (MODE != 2) {
+      if (MODE == 0) __syncthreads();       // every wave has read the old S
+      const float wl = ret_pow(lg, nt);
+      for (int tile = wave; tile < nDT * nCT; tile += RM_THREADS / LMSF_WAVE) {
+        const int dt = tile / nCT, ct = tile % nCT;
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+        if (MODE == 0) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[r] = sS[(dt * 16 + fg * 4 + r) * RM_BS + ct * 16 + fr] * wl;
+        }
+        const float* ap = sk + fg * dq + dt * 16 + fr;       // K^T: row dd, inner index u
+        const float* bp = sv + fg * RM_BS + ct * 16 + fr;
+        const float* wp = sw + fg;
+#pragma unroll 4
+        for (int kk = 0; kk < L; kk += 4)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ap[kk * dq], bp[kk * RM_BS] * wp[kk], acc, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int dd = dt * 16 + fg * 4 + r, c = ct * 16 + fr;
+          if (MODE == 0) sS[dd * RM_BS + c] = acc[r];
+          else if (dd < d && c < nb) gS[(long)dd * dv + e0 + c] = acc[r];
+        }
+      }
+    }
+  }
+  if (MODE == 0) {
+    __syncthreads();
+    for (int i = tid; i < d * nb; i += RM_THREADS) {
+      const int dd = i / nb, c = i % nb;
+      gS[(long)dd * dv + e0 + c] = sS[dd * RM_BS + c];
+    }
+  }
+}
+
+static size_t ret_mfma_smem(int d, int L) {
+  const int d16 = (d + 15) / 16 * 16;
+  return ((size_t)2 * L * (d16 + 4) + (size_t)L * RM_BS + (size_t)L * (L + 4) + (size_t)d16 * RM_BS + L) * sizeof(float);
+}
+
+// tokens of a chunk of the matrix-core form at heads of d; 0: its operands do not fit a workgroup's LDS
+static int ret_mfma_tokens(int d) {
+  for (int L = 64; L >= 16; L /= 2)
+    if (ret_mfma_smem(d, L) <= 128 * 1024) return L;
+  return 0;
+}
+
 // Chunk after chunk of a segment: the chunk's S_0 takes U's place, then S <- g^n S + U (n: the chunk's tokens); at the
 // end S goes to the slot. A thread an entry of one head's S.
 __global__ __launch_bounds__(256) void retention_fold_kernel(float* __restrict__ state, long state_stride,
@@ -251,6 +415,7 @@ static size_t ret_chunk_smem(int d, int L) {
 
 // tokens of a chunk at heads of d (the most for which a workgroup's operands fit its LDS); 0: none do
 extern "C" int lmsf_retention_chunk_tokens(int d) {
+  if (ret_mfma_tokens(d) > 0) return ret_mfma_tokens(d);
   for (int L = 64; L >= 4; L /= 2)
     if (ret_chunk_smem(d, L) <= 128 * 1024) return L;
   return 0;
@@ -301,15 +466,16 @@ extern "C" int lmsf_retention_chunked(const void* q, const void* k, const void* 
   if (n_tokens == 0 || n_segments == 0) return 0;
   const int L = lmsf_retention_chunk_tokens(d);
   LMSF_CHECK(L > 0, "retention: heads of %d entries do not fit a workgroup's LDS", d);
-  const size_t smem = ret_chunk_smem(d, L);
-  const int n_vb = (dv + RET_DVB - 1) / RET_DVB;
+  const bool mfma = ret_mfma_tokens(d) > 0;
+  const size_t smem = mfma ? ret_mfma_smem(d, L) : ret_chunk_smem(d, L);
+  const int n_vb = mfma ? (dv + RM_NB - 1) / RM_NB : (dv + RET_DVB - 1) / RET_DVB;
   LMSF_CHECK(!chunk_base || (long)n_vb * max_chunks <= 65535, "retention: too many chunks");
   const float* log_decay = decay + H;
-#define RET_LAUNCH(T, MODE, GRID)                                                                                    \
+#define RET_LAUNCH_OF(KERNEL, THREADS, T, MODE, GRID)                                                                \
   do {                                                                                                               \
     static size_t reserved = 0;                                                                                      \
     if (smem > 64 * 1024 && smem > reserved) {                                                                       \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(retention_chunk_kernel<T, MODE>),             \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(KERNEL<T, MODE>),                             \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);                     \
       if (e != hipSuccess) {                                                                                         \
         lmsf_set_error("retention: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));                \
@@ -317,10 +483,14 @@ extern "C" int lmsf_retention_chunked(const void* q, const void* k, const void* 
       }                                                                                                              \
       reserved = smem;                                                                                               \
     }                                                                                                                \
-    hipLaunchKernelGGL((retention_chunk_kernel<T, MODE>), GRID, dim3(RET_THREADS), smem, stream, (const T*)q,        \
-                       (const T*)k, (const T*)v, qkv_stride, positions, table, rot, max_pos, log_decay, state,       \
-                       state_stride, seg_starts, state_slots, o_raw, (long)H * dv, H, d, dv, L, kscale, n_vb,        \
-                       chunk_base, entries);                                                                         \
+    hipLaunchKernelGGL((KERNEL<T, MODE>), GRID, dim3(THREADS), smem, stream, (const T*)q, (const T*)k, (const T*)v,  \
+                       qkv_stride, positions, table, rot, max_pos, log_decay, state, state_stride, seg_starts,       \
+                       state_slots, o_raw, (long)H * dv, H, d, dv, L, kscale, n_vb, chunk_base, entries);            \
+  } while (0)
+#define RET_LAUNCH(T, MODE, GRID)                                                                                    \
+  do {                                                                                                               \
+    if (mfma) RET_LAUNCH_OF(retention_chunk_mfma_kernel, RM_THREADS, T, MODE, GRID);                                 \
+    else RET_LAUNCH_OF(retention_chunk_kernel, RET_THREADS, T, MODE, GRID);                                          \
   } while (0)
   if (!chunk_base) {
     dim3 grid(H, n_segments, n_vb);
@@ -338,6 +508,7 @@ extern "C" int lmsf_retention_chunked(const void* q, const void* k, const void* 
     LMSF_LAUNCH_CHECK("retention_chunk (outputs)");
   }
 #undef RET_LAUNCH
+#undef RET_LAUNCH_OF
   if (dtype == LMSF_F32) ret_heads<float>(o_raw, og, og_stride, out, out_stride, n_tokens, H, dv, eps, stream);
   else ret_heads<bf16_t>(o_raw, og, og_stride, out, out_stride, n_tokens, H, dv, eps, stream);
   LMSF_LAUNCH_CHECK("retention_head");
