@@ -63,10 +63,12 @@ def batch_of(lens, slots, first_pos=None, dev="cuda"):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,d,dv,rot,lens", [(3, 8, 20, 4, [5, 1, 17]), (2, 64, 96, 64, [300, 2, 70]), (1, 24, 8, 0, [1, 1, 1]),
-                                              (4, 128, 40, 32, [130, 64]), (2, 20, 33, 20, [16, 47, 200])])
+                                              (4, 128, 40, 32, [130, 64]), (2, 20, 33, 20, [16, 47, 200]),
+                                              (2, 256, 16, 0, [50, 2]), (1, 320, 24, 64, [40, 5])])
 def test_retention_in_all_its_forms_against_the_recurrence(dtype, H, d, dv, rot, lens):
     """Token by token, chunks one after the other and chunks side by side, each segment continued from a state that
-    an earlier step left, against the plain recurrence in float64."""
+    an earlier step left, against the plain recurrence in float64. Heads of up to 256 entries take the matrix-core
+    form of the chunks (64, 32 or 16 tokens a chunk), wider ones the scalar form."""
     o = ops()
     g = torch.Generator().manual_seed(H * 100 + d)
     decay = [1.0, 0.9, 0.5, 0.999][:H]
