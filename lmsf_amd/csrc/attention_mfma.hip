@@ -39,6 +39,21 @@ union Frag8 {
   uint32_t w[4];
 };
 
+// Softmax weights in full float32 for the second product (WP == 3; WP == 1: the weights rounded to bfloat16): a
+// float32 number is exactly the sum of three bfloat16 numbers (8 + 8 + 8 bits), its rounding and twice the rounding
+// of what is left; the matrix cores multiply each part with the values and add up in float32. ``hi`` holds the eight
+// weights pv rounded; the other two parts go to ``rest``.
+__device__ __forceinline__ void weight_parts(const float* pv, const Frag8& hi, Frag8 (&rest)[2]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t w = hi.w[i];
+    const float r0 = pv[2 * i] - __uint_as_float(w << 16), r1 = pv[2 * i + 1] - __uint_as_float(w & 0xffff0000u);
+    const uint32_t mid = pack2_bf16(r0, r1);
+    rest[0].w[i] = mid;
+    rest[1].w[i] = pack2_bf16(r0 - __uint_as_float(mid << 16), r1 - __uint_as_float(mid & 0xffff0000u));
+  }
+}
+
 // Maximum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (the lanes that hold one query row's scores), with
 // gfx950's row and half-wave swaps: two VALU instructions each instead of two trips through LDS.
 // v_permlane16_swap exchanges the odd rows of 16 lanes of its first operand with the even rows of its
@@ -92,7 +107,7 @@ __device__ __forceinline__ long v_col_offset(const KvView& G, int key) {
 // One workgroup of 4 waves per (tile, kv head, block of HB heads of its group). Wave w owns the rows
 // (w * NQB + j) * 16 + c, j < NQB, c = lane % 16; row r is token r / HB of the tile and head r % HB of
 // the block. tiles[2 i], tiles[2 i + 1]: first flat token and number of tokens of tile i.
-template <int DPAD, int NQB>
+template <int DPAD, int NQB, int WP = 1>
 __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables,
@@ -179,6 +194,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     const long vo0 = v_col_offset(G, kbase + 4 * g), vo1 = v_col_offset(G, kbase + 16 + 4 * g);
     // mask, online softmax, probabilities as the B operand of the second product
     Frag8 pf[NQB];
+    Frag8 pr[NQB][2];
 #pragma unroll
     for (int j = 0; j < NQB; ++j) {
       float sv[8];
@@ -212,6 +228,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
       pf[j].w[1] = pack2_bf16(pv[2], pv[3]);
       pf[j].w[2] = pack2_bf16(pv[4], pv[5]);
       pf[j].w[3] = pack2_bf16(pv[6], pv[7]);
+      if constexpr (WP == 3) weight_parts(pv, pf[j], pr[j]);
     }
     // O^T += V^T P^T
 #pragma unroll
@@ -222,7 +239,13 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
         vf.h[0] = *reinterpret_cast<const uint2*>(v_pages + vo0 + dvo);
         vf.h[1] = *reinterpret_cast<const uint2*>(v_pages + vo1 + dvo);
 #pragma unroll
-        for (int j = 0; j < NQB; ++j) acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[j].v, acc[v][j], 0, 0, 0);
+        for (int j = 0; j < NQB; ++j) {
+          acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[j].v, acc[v][j], 0, 0, 0);
+          if constexpr (WP == 3) {
+            acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pr[j][0].v, acc[v][j], 0, 0, 0);
+            acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pr[j][1].v, acc[v][j], 0, 0, 0);
+          }
+        }
       }
     }
   }
@@ -314,7 +337,7 @@ __device__ __forceinline__ unsigned lds_address(const void* p) {
 #define PREFILL_BT_CAP 2048
 #define PREFILL_BT_CAP_SMALL 64
 #define PREFILL_BT_PAD 8
-template <int DPAD, int NQB, int STAGES, int NW>
+template <int DPAD, int NQB, int STAGES, int NW, int WP = 1>
 __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_kernel(
     const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables,
@@ -558,6 +581,7 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
       }
       const bool need_mask = kbase + 31 > wminpos || kbase < wmaxlo;   // the same for the whole wave
       Frag8 pf[NQB];
+      Frag8 pr[NQB][2];
 #pragma unroll
       for (int j = 0; j < NQB; ++j) {
         float r[8];
@@ -601,11 +625,18 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
         pf[j].w[1] = pack2_bf16(pv[2], pv[3]);
         pf[j].w[2] = pack2_bf16(pv[4], pv[5]);
         pf[j].w[3] = pack2_bf16(pv[6], pv[7]);
+        if constexpr (WP == 3) weight_parts(pv, pf[j], pr[j]);
       }
 #pragma unroll
       for (int v = 0; v < DV; ++v)
 #pragma unroll
-        for (int j = 0; j < NQB; ++j) acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pf[j].v, acc[v][j], 0, 0, 0);
+        for (int j = 0; j < NQB; ++j) {
+          acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pf[j].v, acc[v][j], 0, 0, 0);
+          if constexpr (WP == 3) {
+            acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pr[j][0].v, acc[v][j], 0, 0, 0);
+            acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pr[j][1].v, acc[v][j], 0, 0, 0);
+          }
+        }
     }
   };
   for (int it = 0; it < n_steps; it += STAGES) {
@@ -637,7 +668,7 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
 }
 
 
-template <int DPAD>
+template <int DPAD, int WP>
 static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, long q_stride, bf16_t* out,
                               long out_stride, const bf16_t* k_pages, const bf16_t* v_pages, const int* block_tables,
                               int btw, const int* tiles, const int* seg, const int* pos, int nh, int nkv, int d, int ps,
@@ -652,7 +683,7 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
   // waves on every SIMD, which hide each other's waits.
   constexpr int NW = (DPAD == 64 || DPAD == 128) ? 8 : 4;
   const size_t smem = (size_t)STAGES * 4 * 32 * DPAD + (PREFILL_BT_CAP + PREFILL_BT_PAD) * sizeof(int);
-  auto kernel = attn_prefill_dma_kernel<DPAD, 8 / NW, STAGES, NW>;
+  auto kernel = attn_prefill_dma_kernel<DPAD, 8 / NW, STAGES, NW, WP>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -710,7 +741,7 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
 // V page holds and every line is asked for twice: continuous batching at 32 kv heads with pages of 32 tokens 3,580 ->
 // 3,710 generated tokens/s (pages of 16: 3,830), with pages of 64 3,030 -> 3,290; 8 tokens of 8,000 keys at 8 kv heads
 // with pages of 64 1,520 -> 1,770 tokens/s. Pages of 8 and 16 tokens stay with the other dealing (measured above).
-template <int DPAD, bool FULL, bool ROW8>
+template <int DPAD, bool FULL, bool ROW8, int WP = 1>
 __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables, int btw,
@@ -838,11 +869,17 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     pf.w[1] = pack2_bf16(pv[2], pv[3]);
     pf.w[2] = pack2_bf16(pv[4], pv[5]);
     pf.w[3] = pack2_bf16(pv[6], pv[7]);
+    Frag8 pr[2];
+    if constexpr (WP == 3) weight_parts(pv, pf, pr);
 #pragma unroll
     for (int v = 0; v < DV; ++v) {
       if (FULL || v * 16 < d) {
         acc[v] *= corr;
         acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pf.v, acc[v], 0, 0, 0);
+        if constexpr (WP == 3) {
+          acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pr[0].v, acc[v], 0, 0, 0);
+          acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pr[1].v, acc[v], 0, 0, 0);
+        }
       }
     }
   };
@@ -1037,6 +1074,8 @@ extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, v
   if (int rc = check_common("paged_attention_prefill", q, out, k_pages, v_pages, block_tables, seg, pos, q_stride,
                             out_stride, num_pages, btw, nh, nkv, d, ps, window))
     return rc;
+  const bool wp3 = (variant & LMSF_ATTENTION_WEIGHTS_F32) != 0;     // softmax weights in full float32
+  variant &= ~LMSF_ATTENTION_WEIGHTS_F32;
   LMSF_CHECK(tiles != nullptr && n_tiles >= 0, "paged_attention_prefill: bad tile list");
   LMSF_CHECK(scale > 0.f, "paged_attention_prefill: the scale must be positive, got %g", (double)scale);
   if (n_tiles == 0) return 0;
@@ -1049,10 +1088,10 @@ extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, v
     // tiles staged in LDS
     const int bt_cap = variant == 2 ? PREFILL_BT_CAP_SMALL : PREFILL_BT_CAP;
     int rc = 0;
-#define LAUNCH_LDS(DP)                                                                                           \
-  rc = launch_prefill_dma<DP>(grid, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride,                \
-                              (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, btw, tiles, seg, pos, \
-                              nh, nkv, d, ps, scale_log2, window, HB, n_hb, bt_cap)
+#define LDS_ARGS                                                                                                    \
+  grid, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
+      block_tables, btw, tiles, seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, bt_cap
+#define LAUNCH_LDS(DP) rc = wp3 ? launch_prefill_dma<DP, 3>(LDS_ARGS) : launch_prefill_dma<DP, 1>(LDS_ARGS)
     switch (dpad) {
       case 32: LAUNCH_LDS(32); break;
       case 64: LAUNCH_LDS(64); break;
@@ -1064,14 +1103,20 @@ extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, v
       default: LAUNCH_LDS(256); break;
     }
 #undef LAUNCH_LDS
+#undef LDS_ARGS
     if (rc) return rc;
     LMSF_LAUNCH_CHECK("paged_attention_prefill");
     return 0;
   }
-#define LAUNCH(DP)                                                                                                  \
-  hipLaunchKernelGGL((attn_prefill_mfma_kernel<DP, PREFILL_NQB>), grid, block, 0, stream, (const bf16_t*)q, q_stride, \
-                     (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, btw,   \
-                     tiles, seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb)
+#define LAUNCH_W(DP, W)                                                                                             \
+  hipLaunchKernelGGL((attn_prefill_mfma_kernel<DP, PREFILL_NQB, W>), grid, block, 0, stream, (const bf16_t*)q,      \
+                     q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,            \
+                     block_tables, btw, tiles, seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb)
+#define LAUNCH(DP)                \
+  do {                            \
+    if (wp3) LAUNCH_W(DP, 3);     \
+    else LAUNCH_W(DP, 1);         \
+  } while (0)
   switch (dpad) {
     case 32: LAUNCH(32); break;
     case 64: LAUNCH(64); break;
@@ -1083,18 +1128,19 @@ extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, v
     default: LAUNCH(256); break;
   }
 #undef LAUNCH
+#undef LAUNCH_W
   LMSF_LAUNCH_CHECK("paged_attention_prefill");
   return 0;
 }
 
-template <int DPAD, bool FULL, bool ROW8>
+template <int DPAD, bool FULL, bool ROW8, int WP>
 static int launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, long q_stride, const bf16_t* k_pages,
                          const bf16_t* v_pages, const int* block_tables, int btw, const int* tok_idx, const int* seg,
                          const int* pos, int nh, int nkv, int d, int ps, float scale_log2, int window, int HB, int n_hb,
                          int chunk, int n_splits, float* part_o, float* part_ml, bf16_t* out, long out_stride,
                          int heads_first) {
   const size_t smem = (size_t)(4 * 16 * (DPAD + 4) + 128) * sizeof(float);
-  auto kernel = attn_decode_mfma_kernel<DPAD, FULL, ROW8>;
+  auto kernel = attn_decode_mfma_kernel<DPAD, FULL, ROW8, WP>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -1143,6 +1189,8 @@ extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, vo
   // heads and 64 tokens with contexts of 192 to 2,112 keys: 75 us against 64 us with the heads of a token
   // together and the longest contexts first (32 kv heads: 214 against 176); equal contexts: the same from 16
   // tokens on, and 1 us in 12 the other way round at 8 tokens.
+  const bool wp3 = (order & LMSF_ATTENTION_WEIGHTS_F32) != 0;       // softmax weights in full float32
+  order &= ~LMSF_ATTENTION_WEIGHTS_F32;
   const int heads_first = order == 2 || (order == 0 && n >= 16);
   const float scale_log2 = scale * 1.44269504088896340736f;
   const int dpad = (d + 31) / 32 * 32;
@@ -1155,9 +1203,14 @@ extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, vo
       seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, chunk, n_splits, part_o, part_ml, (bf16_t*)out,       \
       out_stride, heads_first
   const bool row8 = ps % 32 == 0;   // (needs pages of a multiple of 8 tokens; chosen from 32 on)
-#define LAUNCH(DP)                                                                                      \
-  rc = d == DP ? (row8 ? launch_decode<DP, true, true>(DECODE_ARGS) : launch_decode<DP, true, false>(DECODE_ARGS)) \
-               : (row8 ? launch_decode<DP, false, true>(DECODE_ARGS) : launch_decode<DP, false, false>(DECODE_ARGS))
+#define LAUNCH_W(DP, W)                                                                                       \
+  rc = d == DP ? (row8 ? launch_decode<DP, true, true, W>(DECODE_ARGS) : launch_decode<DP, true, false, W>(DECODE_ARGS)) \
+               : (row8 ? launch_decode<DP, false, true, W>(DECODE_ARGS) : launch_decode<DP, false, false, W>(DECODE_ARGS))
+#define LAUNCH(DP)                \
+  do {                            \
+    if (wp3) LAUNCH_W(DP, 3);     \
+    else LAUNCH_W(DP, 1);         \
+  } while (0)
   switch (dpad) {
     case 32: LAUNCH(32); break;
     case 64: LAUNCH(64); break;
@@ -1169,6 +1222,7 @@ extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, vo
     default: LAUNCH(256); break;
   }
 #undef LAUNCH
+#undef LAUNCH_W
 #undef DECODE_ARGS
   if (rc) return rc;
   LMSF_LAUNCH_CHECK("paged_attention_decode");

@@ -13,6 +13,10 @@
 
 // dtype codes shared with the Python side
 enum { LMSF_F32 = 0, LMSF_BF16 = 1 };
+// Added to ``variant`` (prefill) or ``order`` (decode) of the matrix-core attention entry points: the softmax weights
+// enter the product with the values in full float32 (three bfloat16 parts, three matrix instructions) instead of
+// rounded to bfloat16.
+#define LMSF_ATTENTION_WEIGHTS_F32 256
 
 typedef uint16_t bf16_t;  // raw bfloat16 bits
 

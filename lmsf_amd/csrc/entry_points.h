@@ -15,6 +15,7 @@ int lmsf_paged_attention_generic(const void* q, long q_stride, void* out, long o
     n_tokens, int nh, int nkv, int d, int ps, float scale, int window, int dtype, hipStream_t stream);
 
 // attention_mfma.hip
+// (``variant`` of the prefill and ``order`` of the decode entry may have LMSF_ATTENTION_WEIGHTS_F32 of common.h added)
 int lmsf_attention_tile_tokens(int nh, int nkv);
 int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, void* out, long out_stride, const void* k_pages,
     const void* v_pages, long num_pages, const int* block_tables, int btw, const int* tiles, int n_tiles, const int*

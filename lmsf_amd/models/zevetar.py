@@ -207,7 +207,7 @@ def build_zevetar_spec(cfg: ZevetarConfig) -> ModelSpec:
             mixer = PartSpec("latent_attention", {
                 "prefix": "mix", "hidden_size": W, "num_heads": m["heads"], "head_dim": m["dim"], "rot_dim": m["rot_dim"],
                 "v_head_dim": m["vdim"], "kv_rank": m["kv_rank"], "q_rank": m["q_rank"], "scale": m["scale"],
-                "eps": cfg.norm_eps, "owns_latent": src is None, "gate_per_entry": True,
+                "eps": cfg.norm_eps, "owns_latent": src is None, "gate_per_entry": True, "weights_f32": True,
                 "window": (m.get("mask") or {}).get("size"), "cache_window": kept[owner],
                 "position": _rotary(m["rot"], m["rot_dim"], "gptj")})
         else:

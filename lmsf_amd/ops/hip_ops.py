@@ -436,10 +436,12 @@ class HipOps:
     def paged_attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                         block_tables: torch.Tensor, seg: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int, d: int,
                         scale: float, window: int = 0, batch=None, kernel: Optional[str] = None,
-                        chunk: int = 0) -> torch.Tensor:
+                        chunk: int = 0, weights_f32: bool = False) -> torch.Tensor:
         """Attention of every query token over the cached keys of its request: those at positions up to its own,
         within the last ``window`` positions if a window is given, or within its own chunk of ``chunk`` positions
-        (chunks counted from position 0 of the request) if a chunk size is given.
+        (chunks counted from position 0 of the request) if a chunk size is given. ``weights_f32``: in a bfloat16 run
+        the softmax weights enter the product with the values in full float32 (as three bfloat16 parts on the
+        matrix cores) instead of rounded to bfloat16; scores, maxima and sums are float32 either way.
 
         ``q`` is [N, >= nh*d] with unit column stride (it may be the fused QKV buffer, of which the
         first nh*d columns are read). ``k_pages`` [pages, nkv, page_size, d], ``v_pages``
@@ -482,12 +484,13 @@ class HipOps:
                 int(window or 0), _code(q.dtype), self._stream()))
             return out
         plan = self._attention_plan(batch, seg, pos, nh, nkv)
+        exact = self.ATTENTION_WEIGHTS_F32 if weights_f32 else 0
         common = (_ptr(k_pages), _ptr(v_pages), num_pages, _ptr(block_tables), block_tables.shape[1])
         if plan.tiles is not None:
             self._check(self.lib.lmsf_paged_attention_prefill_mfma(
                 _ptr(q), q.stride(0), _ptr(out), out.stride(0), *common, _ptr(plan.tiles), plan.n_tiles,
-                _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0), self.prefill_attention_variant,
-                self._stream()))
+                _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0),
+                self.prefill_attention_variant + exact, self._stream()))
         if plan.n_single:
             c_chunk, c_splits = ctypes.c_int(0), ctypes.c_int(0)
             self.lib.lmsf_route_decode_attention(ctypes.byref(self._tun), plan.n_single, nh, nkv, plan.max_context,
@@ -498,8 +501,10 @@ class HipOps:
             self._check(self.lib.lmsf_paged_attention_decode_mfma(
                 _ptr(q), q.stride(0), _ptr(out), out.stride(0), *common, _ptr(plan.single_tokens), plan.n_single,
                 None if plan.token_is_request else _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale),
-                int(window or 0), chunk, n_splits, _ptr(scratch), self.decode_attention_order, self._stream()))
+                int(window or 0), chunk, n_splits, _ptr(scratch), self.decode_attention_order + exact, self._stream()))
         return out
+
+    ATTENTION_WEIGHTS_F32 = 256     # csrc/entry_points.h: LMSF_ATTENTION_WEIGHTS_F32
 
     def _attention_plan(self, batch, seg: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int) -> "_AttentionPlan":
         """How a step's tokens are split between the two matrix-core kernels: requests with one token go

@@ -12,9 +12,11 @@ out_h is multiplied by sigmoid(Wg h)_h before the output projection (one gate a 
 for every entry of every head's value). A layer may read another layer's cache (the schedule's ``cache_from``): it
 then has no down-projection to the latent, only its own up-projections. ``window``: a query sees itself and the
 window - 1 positions before it; ``cache_window`` is what the pages are kept for (the widest window among the layers
-that read them; None: everything). A position encoding of style "gptj" (pairs (2i, 2i + 1)) is served by the same
-kernels: the rows of Wuq and Wdkv that make the rotated entries are put in the order (0, 2, 4, ..., 1, 3, 5, ...) at
-load, which changes no score (the same permutation on both sides of the dot product) and makes the pairs (i, i + rot/2).
+that read them; None: everything). ``weights_f32``: the softmax weights stay float32 into the product with the cached
+rows (``HipOps.paged_attention``), for a design that asks for it. A position encoding of style "gptj" (pairs
+(2i, 2i + 1)) is served by the same kernels: the rows of Wuq and Wdkv that make the rotated entries are put in the order
+(0, 2, 4, ..., 1, 3, 5, ...) at load, which changes no score (the same permutation on both sides of the dot product)
+and makes the pairs (i, i + rot/2).
 
 The reference has no such mixer (its attention keeps full keys and values per kv head,
 core/src/model_executor/layers/attention.rs:91-231).
@@ -57,9 +59,10 @@ class LatentAttention(Mixer):
     def __init__(self, prefix: str, rt: Runtime, hidden_size: int, num_heads: int, head_dim: int, rot_dim: int,
                  v_head_dim: int, kv_rank: int, q_rank: int, scale: float, eps: float, position: PartSpec,
                  owns_latent: bool = True, names: Optional[Dict[str, str]] = None, gate_per_entry: bool = False,
-                 window: Optional[int] = None, cache_window: Optional[int] = None):
+                 window: Optional[int] = None, cache_window: Optional[int] = None, weights_f32: bool = False):
         super().__init__(prefix, rt)
         self.gate_per_entry = bool(gate_per_entry)
+        self.weights_f32 = bool(weights_f32)
         self.window = int(window) if window else None
         self.cache_window = int(cache_window) if cache_window else None
         if self.cache_window is not None and (self.window is None or self.window > self.cache_window):
@@ -130,8 +133,9 @@ class LatentAttention(Mixer):
         # Uk_h^T qn_h -> qa[:, h, :R]; rotate(qr_h) -> qa[:, h, R:R + dr]; zeros behind
         ops.head_linear(q, self.dn + self.dr, self.uk_t.weight, qa, self.D,
                         rope_tail=(self.dn, self.R, self.dr, ctx.positions, table))
+        more = {"weights_f32": True} if self.weights_f32 else {}
         a = ops.paged_attention(qa, binding.k_pages, binding.v_pages, group.block_tables, ctx.seg_of_token,
-                                ctx.positions, self.H, 1, self.D, self.scale, self.window or 0, batch=ctx)
+                                ctx.positions, self.H, 1, self.D, self.scale, self.window or 0, batch=ctx, **more)
         out = torch.empty((N, self.H * self.dv), dtype=q.dtype, device=q.device)
         ops.head_linear(a, self.D, self.uv.weight, out, self.dv, gate=low[:, self.at_gate:], gate_wide=self.gate_per_entry)
         return self.o.forward(out)

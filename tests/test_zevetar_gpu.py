@@ -193,6 +193,41 @@ def test_per_head_products_with_a_gate_for_every_output(dtype, N, H, O, K):
     close(out, want, dtype)
 
 
+@pytest.mark.parametrize("d,ps,ctx,n_query", [(64, 16, 2, 1), (64, 16, 2, 2), (160, 8, 41, 1), (160, 8, 41, 41),
+                                              (256, 4, 300, 1), (128, 16, 700, 130), (48, 32, 90, 3), (96, 4, 50, 50)])
+def test_softmax_weights_in_float32_into_the_product_with_the_values(d, ps, ctx, n_query):
+    """Values of +1 and -1 in turn under nearly equal weights: the result is a small difference of large sums, and what
+    rounding the weights to bfloat16 costs (2^-9 of a weight) stands out against what rounding the result costs (2^-9
+    of the result). With ``weights_f32`` every entry is within the result's own rounding of the float64 value; without
+    it, it is not (which says that the case can tell)."""
+    g = torch.Generator().manual_seed(d + ctx)
+    nh, nkv = 8, 1
+    pages = -(-ctx // ps)
+    k = (torch.randn(pages, nkv, ps, d, generator=g) * 0.3).to(torch.bfloat16)
+    sign = torch.tensor([1.0 if j % 2 == 0 else -1.0 for j in range(pages * ps)]).reshape(pages, 1, 1, ps)
+    v = sign.expand(pages, nkv, d, ps).contiguous().to(torch.bfloat16)
+    q = (torch.randn(n_query, nh * d, generator=g) * 0.05).to(torch.bfloat16)
+    pos = torch.arange(ctx - n_query, ctx, dtype=torch.int32)
+    seg = torch.zeros(n_query, dtype=torch.int32)
+    bt = torch.arange(pages, dtype=torch.int32).reshape(1, pages)
+    scale = d ** -0.5
+    keys = k.double().permute(1, 0, 2, 3).reshape(nkv, pages * ps, d)[0]                     # [keys, d]
+    want = torch.empty(n_query, nh, dtype=torch.float64)
+    for i in range(n_query):
+        n = int(pos[i]) + 1
+        sc = (q[i].double().reshape(nh, d) @ keys[:n].T) * scale
+        want[i] = (torch.softmax(sc, -1) * sign.reshape(-1)[:n].double()).sum(-1)
+    errs = {}
+    for exact in (True, False):
+        got = ops().paged_attention(q.cuda(), k.cuda(), v.cuda(), bt.cuda(), seg.cuda(), pos.cuda(), nh, nkv, d, scale, 0,
+                                    kernel="mfma", weights_f32=exact).cpu().double().reshape(n_query, nh, d)
+        assert float((got - got[:, :, :1]).abs().max()) == 0.0           # every column of V is the same
+        errs[exact] = (got[:, :, 0] - want).abs()
+    bound = 2.0 ** -8 * want.abs() + 3e-6
+    assert bool((errs[True] <= bound).all()), float((errs[True] / bound).max())
+    assert float((errs[False] / bound).max()) > 3.0
+
+
 # ---------------------------------------------------------------- through the engine
 
 

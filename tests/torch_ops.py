@@ -125,7 +125,7 @@ class TorchOps:
 
     # ------------------------------------------------------------ attention
     def paged_attention(self, q, k_pages, v_pages, block_tables, seg, pos, nh, nkv, d, scale, window=0, batch=None,
-                        kernel=None, chunk=0):
+                        kernel=None, chunk=0, weights_f32=False):
         N = q.shape[0]
         ps = k_pages.shape[2]
         out = torch.empty((N, nh * d), dtype=q.dtype, device=q.device)
