@@ -92,6 +92,14 @@ class CacheStorage:
         self.bindings = bindings
         self.has_state = any(b.state is not None for b in bindings)
         model.bind_cache(bindings)
+        # an embedding with per-request state (the token before a step's first) gets a row per slot and the spare one
+        # too; it is not cleared when a request takes a slot: such a part tells a request's first token by its position
+        self.embedding_state: Optional[torch.Tensor] = None
+        espec = model.embedding_state() if hasattr(model, "embedding_state") else None
+        if espec is not None:
+            self.embedding_state = torch.zeros((self.num_state_slots + 1,) + tuple(espec.shape), dtype=espec.dtype,
+                                               device=rt.device)
+            model.embedding.bind_state(self.embedding_state)
 
     def clear_state_slots(self, slots: Sequence[int]) -> None:
         """Zeroes these slots of every state tensor: a request that takes a slot finds no trace of the one that
@@ -112,6 +120,8 @@ class CacheStorage:
                 if t is not None and t.data_ptr() not in seen:
                     seen.add(t.data_ptr())
                     total += t.numel() * t.element_size()
+        if self.embedding_state is not None:
+            total += self.embedding_state.numel() * self.embedding_state.element_size()
         return total
 
 

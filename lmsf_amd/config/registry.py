@@ -84,4 +84,8 @@ def load_model_config(folder: str) -> Tuple[Architecture, ArchConfig]:
     """Read ``folder``/config.json and parse it with the class its architecture registered."""
     d = read_config_json(folder)
     arch = resolve_architecture(d)
+    # an architecture some of whose sizes only its tensors' shapes give reads them from the checkpoint's header
+    complete = getattr(arch.config_class, "complete_from_checkpoint", None)
+    if complete is not None:
+        d = complete(d, folder)
     return arch, arch.config_class.from_dict(d)

@@ -29,7 +29,7 @@ template <typename T>
 __global__ __launch_bounds__(GEN_THREADS) void paged_attention_generic_kernel(
     const T* __restrict__ q, long q_stride, T* __restrict__ out, long out_stride, const T* __restrict__ k_pages,
     const T* __restrict__ v_pages, const int* __restrict__ block_tables, int bt_width, const int* __restrict__ seg,
-    const int* __restrict__ pos, int nh, int nkv, int d, int ps, float scale, int window) {
+    const int* __restrict__ pos, int nh, int nkv, int d, int ps, float scale, int window, float softcap) {
   extern __shared__ float smem[];
   float* sq = smem;                       // [d] query, pre-scaled
   float* sp = sq + d;                     // [256] scores, then probabilities
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(GEN_THREADS) void paged_attention_generic_kernel(
         dot += sq[i] * to_f32<T>(kr[i]) + sq[i + 1] * to_f32<T>(kr[i + 1]) + sq[i + 2] * to_f32<T>(kr[i + 2]) +
                sq[i + 3] * to_f32<T>(kr[i + 3]);
       }
-      sc = dot;
+      sc = softcap > 0.f ? softcap * tanhf(dot / softcap) : dot;   // scores bounded by cap tanh(s / cap)
     }
     const float cmax = block_max(sc, red);
     const float m_new = fmaxf(m, cmax);
@@ -113,11 +113,14 @@ __global__ __launch_bounds__(GEN_THREADS) void paged_attention_generic_kernel(
   }
 }
 
-extern "C" int lmsf_paged_attention_generic(const void* q, long q_stride, void* out, long out_stride,
-                                            const void* k_pages, const void* v_pages, long num_pages,
-                                            const int* block_tables, int bt_width, const int* seg, const int* pos,
-                                            int n_tokens, int nh, int nkv, int d, int ps, float scale, int window,
-                                            int dtype, hipStream_t stream) {
+// ``softcap`` c > 0: a score s (after the scale) becomes c tanh(s / c) before the softmax; 0: scores as they are.
+extern "C" int lmsf_paged_attention_generic_capped(const void* q, long q_stride, void* out, long out_stride,
+                                                   const void* k_pages, const void* v_pages, long num_pages,
+                                                   const int* block_tables, int bt_width, const int* seg,
+                                                   const int* pos, int n_tokens, int nh, int nkv, int d, int ps,
+                                                   float scale, int window, float softcap, int dtype,
+                                                   hipStream_t stream) {
+  LMSF_CHECK(softcap >= 0.f, "paged_attention: the soft cap must be >= 0, got %g", (double)softcap);
   LMSF_CHECK(q && out && k_pages && v_pages && block_tables && seg && pos, "paged_attention: null pointer");
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "paged_attention: unknown dtype code %d", dtype);
   LMSF_CHECK(nh > 0 && nkv > 0 && nh % nkv == 0, "paged_attention: heads %d not a multiple of kv heads %d", nh, nkv);
@@ -132,11 +135,21 @@ extern "C" int lmsf_paged_attention_generic(const void* q, long q_stride, void* 
   if (dtype == LMSF_F32)
     hipLaunchKernelGGL((paged_attention_generic_kernel<float>), grid, block, smem, stream, (const float*)q, q_stride,
                        (float*)out, out_stride, (const float*)k_pages, (const float*)v_pages, block_tables, bt_width,
-                       seg, pos, nh, nkv, d, ps, scale, window);
+                       seg, pos, nh, nkv, d, ps, scale, window, softcap);
   else
     hipLaunchKernelGGL((paged_attention_generic_kernel<bf16_t>), grid, block, smem, stream, (const bf16_t*)q, q_stride,
                        (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables,
-                       bt_width, seg, pos, nh, nkv, d, ps, scale, window);
+                       bt_width, seg, pos, nh, nkv, d, ps, scale, window, softcap);
   LMSF_LAUNCH_CHECK("paged_attention_generic");
   return 0;
+}
+
+extern "C" int lmsf_paged_attention_generic(const void* q, long q_stride, void* out, long out_stride,
+                                            const void* k_pages, const void* v_pages, long num_pages,
+                                            const int* block_tables, int bt_width, const int* seg, const int* pos,
+                                            int n_tokens, int nh, int nkv, int d, int ps, float scale, int window,
+                                            int dtype, hipStream_t stream) {
+  return lmsf_paged_attention_generic_capped(q, q_stride, out, out_stride, k_pages, v_pages, num_pages, block_tables,
+                                             bt_width, seg, pos, n_tokens, nh, nkv, d, ps, scale, window, 0.f, dtype,
+                                             stream);
 }

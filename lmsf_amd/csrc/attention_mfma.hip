@@ -104,6 +104,16 @@ __device__ __forceinline__ long v_col_offset(const KvView& G, int key) {
 
 // ---------------------------------------------------------------- prefill
 
+// Scores bounded before the softmax: a raw score r (before the scale) becomes c tanh(r / c) with c = cap / scale, so
+// that the scaled score is cap tanh(scale r / cap); c = 0: scores as they are. tanh x = 1 - 2 / (2^(2 x log2 e) + 1),
+// the hardware's 2^x and reciprocal: good to a few float32 steps, far inside what a bfloat16 run keeps.
+// Callers put one test of c around all the scores of a step, so that attention without a cap pays one branch a step.
+__device__ __forceinline__ float capped_score(float r, float cap_raw) {
+  const float e = __builtin_amdgcn_exp2f(r * (2.88539008177792681472f / cap_raw));
+  return cap_raw * (1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f));
+}
+
+
 // One workgroup of 4 waves per (tile, kv head, block of HB heads of its group). Wave w owns the rows
 // (w * NQB + j) * 16 + c, j < NQB, c = lane % 16; row r is token r / HB of the tile and head r % HB of
 // the block. tiles[2 i], tiles[2 i + 1]: first flat token and number of tokens of tile i.
@@ -112,7 +122,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables,
     int btw, const int* __restrict__ tiles, const int* __restrict__ seg, const int* __restrict__ pos, int nh, int nkv,
-    int d, int ps, float scale_log2, int window, int HB, int n_hb) {
+    int d, int ps, float scale_log2, float cap_raw, int window, int HB, int n_hb) {
   constexpr int DS = DPAD / 32, DV = DPAD / 16;
   const int tile = blockIdx.x;
   const int kvh = blockIdx.y / n_hb, hb = blockIdx.y - kvh * n_hb;
@@ -199,6 +209,12 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     for (int j = 0; j < NQB; ++j) {
       float sv[8];
       float mx = -INFINITY;
+      if (cap_raw > 0.f) {
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) st[b][j][i] = capped_score(st[b][j][i], cap_raw);
+      }
 #pragma unroll
       for (int b = 0; b < 2; ++b)
 #pragma unroll
@@ -342,7 +358,7 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
     const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables,
     int btw, const int* __restrict__ tiles, const int* __restrict__ seg, const int* __restrict__ pos, int nh, int nkv,
-    int d, int ps_log2, float scale_log2, int window, int HB, int n_hb, int bt_cap, int n_cus) {
+    int d, int ps_log2, float scale_log2, float cap_raw, int window, int HB, int n_hb, int bt_cap, int n_cus) {
   constexpr int DS = DPAD / 32, DV = DPAD / 16;
   constexpr int PR = DPAD / 8;                   // 16-byte pieces per K row
   constexpr bool PR_POW2 = (PR & (PR - 1)) == 0;
@@ -589,6 +605,10 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
         for (int b = 0; b < 2; ++b)
 #pragma unroll
           for (int i = 0; i < 4; ++i) r[b * 4 + i] = st[b][j][i];
+        if (__builtin_expect(cap_raw > 0.f, 0)) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) r[e] = capped_score(r[e], cap_raw);
+        }
         if (need_mask) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
@@ -672,7 +692,7 @@ template <int DPAD, int WP>
 static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, long q_stride, bf16_t* out,
                               long out_stride, const bf16_t* k_pages, const bf16_t* v_pages, const int* block_tables,
                               int btw, const int* tiles, const int* seg, const int* pos, int nh, int nkv, int d, int ps,
-                              float scale_log2, int window, int HB, int n_hb, int bt_cap) {
+                              float scale_log2, float cap_raw, int window, int HB, int n_hb, int bt_cap) {
   int ps_log2 = 0;
   while ((1 << ps_log2) < ps) ++ps_log2;
   // four stages of a head size of 128 and the table are 72 KB: two workgroups share a compute unit's LDS,
@@ -695,7 +715,7 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
     configured = true;
   }
   hipLaunchKernelGGL(kernel, dim3(grid.x * grid.y), dim3(NW * 64), smem, stream, q, q_stride, out, out_stride, k_pages,
-                     v_pages, block_tables, btw, tiles, seg, pos, nh, nkv, d, ps_log2, scale_log2, window, HB, n_hb,
+                     v_pages, block_tables, btw, tiles, seg, pos, nh, nkv, d, ps_log2, scale_log2, cap_raw, window, HB, n_hb,
                      bt_cap, lmsf_compute_units());
   return 0;
 }
@@ -746,7 +766,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables, int btw,
     const int* __restrict__ tok_idx, const int* __restrict__ seg, const int* __restrict__ pos, int nh, int nkv, int d,
-    int ps, float scale_log2, int window, int HB, int n_hb, int chunk, int n_splits, float* __restrict__ part_o,
+    int ps, float scale_log2, float cap_raw, int window, int HB, int n_hb, int chunk, int n_splits, float* __restrict__ part_o,
     float* __restrict__ part_ml, bf16_t* __restrict__ out, long out_stride, int heads_first) {
   constexpr int DS = DPAD / 32, DV = DPAD / 16;
   extern __shared__ float lds_f[];
@@ -843,6 +863,10 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
       f32x4_t a = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < DS; ++s) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[b][s].v, qf[s].v, a, 0, 0, 0);
+      if (cap_raw > 0.f) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] = capped_score(a[i], cap_raw);
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int key = ROW8 ? kbase + 8 * g + 4 * b + i : kbase + b * 16 + g * 4 + i;
@@ -1066,11 +1090,15 @@ extern "C" int lmsf_attention_tile_tokens(int nh, int nkv) {
 // of a tile belong to one request and stand at consecutive positions. variant 0: keys and values staged in
 // LDS where the page size allows it (the default); 1: every wave fetches them itself; 2: as 0 with a window of 64
 // entries of the block table in LDS instead of 2,048, so that it moves at contexts that a test can afford.
-extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, void* out, long out_stride,
-                                                 const void* k_pages, const void* v_pages, long num_pages,
-                                                 const int* block_tables, int btw, const int* tiles, int n_tiles,
-                                                 const int* seg, const int* pos, int nh, int nkv, int d, int ps,
-                                                 float scale, int window, int variant, hipStream_t stream) {
+// ``softcap`` c > 0: a scaled score s becomes c tanh(s / c) before the softmax; 0: scores as they are.
+extern "C" int lmsf_paged_attention_prefill_mfma_capped(const void* q, long q_stride, void* out, long out_stride,
+                                                        const void* k_pages, const void* v_pages, long num_pages,
+                                                        const int* block_tables, int btw, const int* tiles,
+                                                        int n_tiles, const int* seg, const int* pos, int nh, int nkv,
+                                                        int d, int ps, float scale, int window, float softcap,
+                                                        int variant, hipStream_t stream) {
+  LMSF_CHECK(softcap >= 0.f, "paged_attention_prefill: the soft cap must be >= 0, got %g", (double)softcap);
+  const float cap_raw = softcap > 0.f ? softcap / scale : 0.f;
   if (int rc = check_common("paged_attention_prefill", q, out, k_pages, v_pages, block_tables, seg, pos, q_stride,
                             out_stride, num_pages, btw, nh, nkv, d, ps, window))
     return rc;
@@ -1090,7 +1118,7 @@ extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, v
     int rc = 0;
 #define LDS_ARGS                                                                                                    \
   grid, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
-      block_tables, btw, tiles, seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, bt_cap
+      block_tables, btw, tiles, seg, pos, nh, nkv, d, ps, scale_log2, cap_raw, window, HB, n_hb, bt_cap
 #define LAUNCH_LDS(DP) rc = wp3 ? launch_prefill_dma<DP, 3>(LDS_ARGS) : launch_prefill_dma<DP, 1>(LDS_ARGS)
     switch (dpad) {
       case 32: LAUNCH_LDS(32); break;
@@ -1111,7 +1139,7 @@ extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, v
 #define LAUNCH_W(DP, W)                                                                                             \
   hipLaunchKernelGGL((attn_prefill_mfma_kernel<DP, PREFILL_NQB, W>), grid, block, 0, stream, (const bf16_t*)q,      \
                      q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages,            \
-                     block_tables, btw, tiles, seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb)
+                     block_tables, btw, tiles, seg, pos, nh, nkv, d, ps, scale_log2, cap_raw, window, HB, n_hb)
 #define LAUNCH(DP)                \
   do {                            \
     if (wp3) LAUNCH_W(DP, 3);     \
@@ -1136,7 +1164,7 @@ extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, v
 template <int DPAD, bool FULL, bool ROW8, int WP>
 static int launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, long q_stride, const bf16_t* k_pages,
                          const bf16_t* v_pages, const int* block_tables, int btw, const int* tok_idx, const int* seg,
-                         const int* pos, int nh, int nkv, int d, int ps, float scale_log2, int window, int HB, int n_hb,
+                         const int* pos, int nh, int nkv, int d, int ps, float scale_log2, float cap_raw, int window, int HB, int n_hb,
                          int chunk, int n_splits, float* part_o, float* part_ml, bf16_t* out, long out_stride,
                          int heads_first) {
   const size_t smem = (size_t)(4 * 16 * (DPAD + 4) + 128) * sizeof(float);
@@ -1152,7 +1180,7 @@ static int launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, long q_
     configured = true;
   }
   hipLaunchKernelGGL(kernel, grid, dim3(256), smem, stream, q, q_stride, k_pages, v_pages, block_tables, btw, tok_idx,
-                     seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, chunk, n_splits, part_o, part_ml, out,
+                     seg, pos, nh, nkv, d, ps, scale_log2, cap_raw, window, HB, n_hb, chunk, n_splits, part_o, part_ml, out,
                      out_stride, heads_first);
   return 0;
 }
@@ -1168,12 +1196,14 @@ extern "C" long lmsf_attention_decode_scratch_floats(int n, int nh, int d, int n
 // n_splits * chunk must cover the longest context. scratch: lmsf_attention_decode_scratch_floats floats
 // (not touched with n_splits == 1). seg null: token i is the only token of request i (row i of the block tables),
 // as in a step of single tokens.
-extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, void* out, long out_stride,
-                                                const void* k_pages, const void* v_pages, long num_pages,
-                                                const int* block_tables, int btw, const int* tok_idx, int n,
-                                                const int* seg, const int* pos, int nh, int nkv, int d, int ps,
-                                                float scale, int window, int chunk, int n_splits, float* scratch,
-                                                int order, hipStream_t stream) {
+extern "C" int lmsf_paged_attention_decode_mfma_capped(const void* q, long q_stride, void* out, long out_stride,
+                                                       const void* k_pages, const void* v_pages, long num_pages,
+                                                       const int* block_tables, int btw, const int* tok_idx, int n,
+                                                       const int* seg, const int* pos, int nh, int nkv, int d, int ps,
+                                                       float scale, int window, float softcap, int chunk, int n_splits,
+                                                       float* scratch, int order, hipStream_t stream) {
+  LMSF_CHECK(softcap >= 0.f && scale > 0.f, "paged_attention_decode: the soft cap must be >= 0 and the scale positive");
+  const float cap_raw = softcap > 0.f ? softcap / scale : 0.f;
   if (int rc = check_common("paged_attention_decode", q, out, k_pages, v_pages, block_tables, seg ? seg : pos, pos,
                             q_stride, out_stride, num_pages, btw, nh, nkv, d, ps, window))
     return rc;
@@ -1200,7 +1230,7 @@ extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, vo
   int rc = 0;
 #define DECODE_ARGS                                                                                                 \
   grid, stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, btw, tok_idx, \
-      seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, chunk, n_splits, part_o, part_ml, (bf16_t*)out,       \
+      seg, pos, nh, nkv, d, ps, scale_log2, cap_raw, window, HB, n_hb, chunk, n_splits, part_o, part_ml, (bf16_t*)out,       \
       out_stride, heads_first
   const bool row8 = ps % 32 == 0;   // (needs pages of a multiple of 8 tokens; chosen from 32 on)
 #define LAUNCH_W(DP, W)                                                                                       \
@@ -1235,4 +1265,25 @@ extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, vo
                      out_stride, tok_idx, pos, nh, d, window, chunk, n_splits);
   LMSF_LAUNCH_CHECK("paged_attention_decode_reduce");
   return 0;
+}
+
+extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, void* out, long out_stride,
+                                                 const void* k_pages, const void* v_pages, long num_pages,
+                                                 const int* block_tables, int btw, const int* tiles, int n_tiles,
+                                                 const int* seg, const int* pos, int nh, int nkv, int d, int ps,
+                                                 float scale, int window, int variant, hipStream_t stream) {
+  return lmsf_paged_attention_prefill_mfma_capped(q, q_stride, out, out_stride, k_pages, v_pages, num_pages,
+                                                  block_tables, btw, tiles, n_tiles, seg, pos, nh, nkv, d, ps, scale,
+                                                  window, 0.f, variant, stream);
+}
+
+extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, void* out, long out_stride,
+                                                const void* k_pages, const void* v_pages, long num_pages,
+                                                const int* block_tables, int btw, const int* tok_idx, int n,
+                                                const int* seg, const int* pos, int nh, int nkv, int d, int ps,
+                                                float scale, int window, int chunk, int n_splits, float* scratch,
+                                                int order, hipStream_t stream) {
+  return lmsf_paged_attention_decode_mfma_capped(q, q_stride, out, out_stride, k_pages, v_pages, num_pages,
+                                                 block_tables, btw, tok_idx, n, seg, pos, nh, nkv, d, ps, scale,
+                                                 window, 0.f, chunk, n_splits, scratch, order, stream);
 }

@@ -63,7 +63,7 @@ template <typename T>
 __global__ __launch_bounds__(MOE_THREADS) void moe_gate_up_kernel(
     const T* __restrict__ h, long h_stride, const T* __restrict__ Wgu, const int* __restrict__ ids,
     const int* __restrict__ table, int vocab, int top, int E, T* __restrict__ act, int F, int W, int vec,
-    const float* __restrict__ pair_scale) {
+    const float* __restrict__ pair_scale, int gated) {
   extern __shared__ float sh[];   // [W]
   const int nk = blockIdx.x, n = nk / top, k = nk - n * top;
   const int id = min(max(ids ? ids[n] : n, 0), vocab - 1);
@@ -73,11 +73,22 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gate_up_kernel(
   __syncthreads();
   const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
   const int f0 = (blockIdx.y * MOE_WAVES + wave) * MOE_OUT_PER_WAVE;
-  const T* We = Wgu + (long)e * 2 * F * W;
+  const T* We = Wgu + (long)e * (gated ? 2 : 1) * F * W;
   if (f0 >= F) return;
   const int valid = min(MOE_OUT_PER_WAVE, F - f0);
   float ag[MOE_OUT_PER_WAVE], au[MOE_OUT_PER_WAVE];
   moe_rows_dot<T, MOE_OUT_PER_WAVE>(We + (long)f0 * W, W, valid, sh, W, lane, vec, ag);
+  if (!gated) {
+    // one matrix an expert: act = relu(W_up h)^2, the product rounded as a stored activation is
+    if (lane < valid) {
+      float uu = 0.f;
+#pragma unroll
+      for (int r = 0; r < MOE_OUT_PER_WAVE; ++r)
+        if (r == lane) uu = fmaxf(to_f32<T>(from_f32<T>(ag[r])), 0.f);
+      act[(long)nk * F + f0 + lane] = from_f32<T>(uu * uu);
+    }
+    return;
+  }
   moe_rows_dot<T, MOE_OUT_PER_WAVE>(We + (long)(F + f0) * W, W, valid, sh, W, lane, vec, au);
   if (lane < valid) {
     // the two products are rounded as stored activations are, then the activation in float32
@@ -97,7 +108,8 @@ template <typename T>
 __global__ __launch_bounds__(MOE_THREADS) void moe_down_kernel(
     const T* __restrict__ act, const T* __restrict__ Wd, const int* __restrict__ ids, const int* __restrict__ table,
     int vocab, int top, int E, float weight, const T* __restrict__ base, long base_stride, T* __restrict__ out,
-    long out_stride, int F, int W, int vec, const float* __restrict__ base_scale) {
+    long out_stride, int F, int W, int vec, const float* __restrict__ base_scale,
+    const float* __restrict__ out_scale) {
   extern __shared__ float sa[];   // [top, F]
   const int n = blockIdx.x;
   const int id = min(max(ids ? ids[n] : n, 0), vocab - 1);
@@ -113,9 +125,10 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_down_kernel(
   for (int k = 0; k < top; ++k) {
     const int e = min(max(table[(long)id * top + k], 0), E - 1);
     float part[MOE_OUT_PER_WAVE];
+    const float os = out_scale ? out_scale[(long)n * top + k] : 1.f;
     moe_rows_dot<T, MOE_OUT_PER_WAVE>(Wd + ((long)e * W + o0) * F, F, valid, sa + k * F, F, lane, vec, part);
 #pragma unroll
-    for (int r = 0; r < MOE_OUT_PER_WAVE; ++r) total[r] += part[r];
+    for (int r = 0; r < MOE_OUT_PER_WAVE; ++r) total[r] += os * part[r];
   }
   if (lane < valid) {
     float mine = 0.f;
@@ -182,12 +195,14 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
 // at every number of pairs: 2,048 tokens (256 pairs an expert) 319 against 194 us for the four kernels, 512 tokens 230
 // against 98, 64 tokens (8 pairs an expert, every tile mostly empty) 101 against 83.
 
-template <bool GATED>
+// KIND 0: the down product; 1: gate and up with silu(gate) * up; 2: one matrix an expert (Wm [E, O, K]) with relu(.)^2.
+template <int KIND>
 __global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restrict__ x, long x_stride, int top,
                                                            const bf16_t* __restrict__ Wm, const int* __restrict__ order,
                                                            const int* __restrict__ tiles, const int* __restrict__ n_tiles,
                                                            void* __restrict__ y, int O, int K,
                                                            const float* __restrict__ pair_scale) {
+  constexpr bool GATED = KIND == 1, UP = KIND != 0;
   constexpr int AR = GATED ? 256 : 128;            // rows of W a step
   constexpr int NLA = AR * 4 / 256;                // 16-byte pieces of W a thread copies a step
   constexpr int NLB = MOE_TILE * 4 / 256;      // and of the pairs' rows
@@ -213,7 +228,7 @@ __global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restr
 #pragma unroll
   for (int i = 0; i < NLB; ++i) {
     const int p = order[place + min(tid / 4 + i * 64, count - 1)];
-    gb[i] = x + (long)(GATED ? p / top : p) * x_stride + (tid % 4) * 8;
+    gb[i] = x + (long)(UP ? p / top : p) * x_stride + (tid % 4) * 8;
   }
   f32x4_t acc[NA][4];
 #pragma unroll
@@ -270,7 +285,7 @@ __global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restr
     const int slot = wr * 64 + mt * 16 + fr;
     if (slot >= count) continue;
     const int p = order[place + slot];
-    const float ps = GATED && pair_scale ? pair_scale[p] : 1.f;
+    const float ps = UP && pair_scale ? pair_scale[p] : 1.f;
 #pragma unroll
     for (int a = 0; a < 4; ++a)
 #pragma unroll
@@ -280,6 +295,9 @@ __global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restr
         if (GATED) {
           const float g = bf16_to_f32(f32_to_bf16(ps * acc[a][mt][j])), u = bf16_to_f32(f32_to_bf16(ps * acc[NA - 4 + a][mt][j]));
           reinterpret_cast<bf16_t*>(y)[(long)p * O + o] = f32_to_bf16(g / (1.f + expf(-g)) * u);
+        } else if (UP) {
+          const float u = fmaxf(bf16_to_f32(f32_to_bf16(ps * acc[a][mt][j])), 0.f);
+          reinterpret_cast<bf16_t*>(y)[(long)p * O + o] = f32_to_bf16(u * u);
         } else {
           reinterpret_cast<float*>(y)[(long)p * O + o] = acc[a][mt][j];
         }
@@ -291,12 +309,14 @@ __global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restr
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ rows, int top, float weight,
                                                           const bf16_t* __restrict__ base, long base_stride,
                                                           bf16_t* __restrict__ out, long out_stride, int W,
-                                                          const float* __restrict__ base_scale) {
+                                                          const float* __restrict__ base_scale,
+                                                          const float* __restrict__ out_scale) {
   const int n = blockIdx.x;
   const float bs = base_scale ? base_scale[n] : 1.f;
   for (int o = threadIdx.x; o < W; o += 256) {
     float s = 0.f;
-    for (int k = 0; k < top; ++k) s += rows[((long)n * top + k) * W + o];
+    for (int k = 0; k < top; ++k)
+      s += (out_scale ? out_scale[(long)n * top + k] : 1.f) * rows[((long)n * top + k) * W + o];
     const float b = base ? bs * bf16_to_f32(base[(long)n * base_stride + o]) : 0.f;
     out[(long)n * out_stride + o] = f32_to_bf16(b + weight * s);
   }
@@ -315,11 +335,16 @@ extern "C" int lmsf_table_moe_grouped(int dtype, int n_tokens, int top, int E, i
          E <= 4096;
 }
 
-extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const void* Wgu, const void* Wd, const int* ids,
-                              const int* table, int vocab, int top, int E, float weight, const void* base,
-                              long base_stride, const float* pair_scale, const float* base_scale, void* act, void* out,
-                              long out_stride, int n_tokens, int F, int W, int* scratch_ints, float* scratch_rows,
-                              hipStream_t stream) {
+// ``act_kind`` 0: gated experts, Wgu [E, 2 F, W]; 1: experts of one matrix, Wgu [E, F, W], y_e(h) = Wd_e relu(Wu_e h)^2.
+// ``out_scale``: a float32 factor per (token, choice) on what the expert returns (null: none).
+extern "C" int lmsf_table_moe_act(const void* h, int dtype, long h_stride, const void* Wgu, const void* Wd,
+                                  const int* ids, const int* table, int vocab, int top, int E, float weight,
+                                  const void* base, long base_stride, const float* pair_scale,
+                                  const float* base_scale, const float* out_scale, int act_kind, void* act, void* out,
+                                  long out_stride, int n_tokens, int F, int W, int* scratch_ints,
+                                  float* scratch_rows, hipStream_t stream) {
+  LMSF_CHECK(act_kind == 0 || act_kind == 1, "table_moe: unknown kind of expert %d", act_kind);
+  const int gated = act_kind == 0;
   LMSF_CHECK(h && Wgu && Wd && table && act && out, "table_moe: null pointer");
   LMSF_CHECK(ids || vocab >= n_tokens, "table_moe: without token ids the table has a row per token");
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "table_moe: unknown dtype code %d", dtype);
@@ -336,13 +361,17 @@ extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const voi
     int* n_tiles = tiles + 3 * (max_tiles + 1);
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)3 * E * 4, stream, ids, table, vocab, top, E, P,
                        MOE_TILE, order, tiles, n_tiles);
-    hipLaunchKernelGGL((moe_tile_lds_kernel<true>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream,
-                       (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W, pair_scale);
-    hipLaunchKernelGGL((moe_tile_lds_kernel<false>), dim3(max_tiles, (W + 127) / 128), dim3(256), 0, stream,
+    if (gated)
+      hipLaunchKernelGGL((moe_tile_lds_kernel<1>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream,
+                         (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W, pair_scale);
+    else
+      hipLaunchKernelGGL((moe_tile_lds_kernel<2>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream,
+                         (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W, pair_scale);
+    hipLaunchKernelGGL((moe_tile_lds_kernel<0>), dim3(max_tiles, (W + 127) / 128), dim3(256), 0, stream,
                        (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows, W,
                        F, (const float*)nullptr);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(256), 0, stream, scratch_rows, top, weight,
-                       (const bf16_t*)base, base_stride, (bf16_t*)out, out_stride, W, base_scale);
+                       (const bf16_t*)base, base_stride, (bf16_t*)out, out_stride, W, base_scale, out_scale);
     LMSF_LAUNCH_CHECK("table_moe (grouped)");
     return 0;
   }
@@ -352,19 +381,29 @@ extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const voi
   const int vec1 = W % vn == 0 && lmsf_aligned16(Wgu), vec2 = F % vn == 0 && lmsf_aligned16(Wd);
   if (dtype == LMSF_F32) {
     hipLaunchKernelGGL((moe_gate_up_kernel<float>), g1, dim3(MOE_THREADS), (size_t)W * 4, stream, (const float*)h,
-                       h_stride, (const float*)Wgu, ids, table, vocab, top, E, (float*)act, F, W, vec1, pair_scale);
+                       h_stride, (const float*)Wgu, ids, table, vocab, top, E, (float*)act, F, W, vec1, pair_scale, gated);
     hipLaunchKernelGGL((moe_down_kernel<float>), g2, dim3(MOE_THREADS), (size_t)top * F * 4, stream, (const float*)act,
                        (const float*)Wd, ids, table, vocab, top, E, weight, (const float*)base, base_stride,
-                       (float*)out, out_stride, F, W, vec2, base_scale);
+                       (float*)out, out_stride, F, W, vec2, base_scale, out_scale);
   } else {
     hipLaunchKernelGGL((moe_gate_up_kernel<bf16_t>), g1, dim3(MOE_THREADS), (size_t)W * 4, stream, (const bf16_t*)h,
-                       h_stride, (const bf16_t*)Wgu, ids, table, vocab, top, E, (bf16_t*)act, F, W, vec1, pair_scale);
+                       h_stride, (const bf16_t*)Wgu, ids, table, vocab, top, E, (bf16_t*)act, F, W, vec1, pair_scale, gated);
     hipLaunchKernelGGL((moe_down_kernel<bf16_t>), g2, dim3(MOE_THREADS), (size_t)top * F * 4, stream,
                        (const bf16_t*)act, (const bf16_t*)Wd, ids, table, vocab, top, E, weight, (const bf16_t*)base,
-                       base_stride, (bf16_t*)out, out_stride, F, W, vec2, base_scale);
+                       base_stride, (bf16_t*)out, out_stride, F, W, vec2, base_scale, out_scale);
   }
   LMSF_LAUNCH_CHECK("table_moe");
   return 0;
+}
+
+extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const void* Wgu, const void* Wd, const int* ids,
+                              const int* table, int vocab, int top, int E, float weight, const void* base,
+                              long base_stride, const float* pair_scale, const float* base_scale, void* act, void* out,
+                              long out_stride, int n_tokens, int F, int W, int* scratch_ints, float* scratch_rows,
+                              hipStream_t stream) {
+  return lmsf_table_moe_act(h, dtype, h_stride, Wgu, Wd, ids, table, vocab, top, E, weight, base, base_stride,
+                            pair_scale, base_scale, nullptr, 0, act, out, out_stride, n_tokens, F, W, scratch_ints,
+                            scratch_rows, stream);
 }
 
 // ---------------------------------------------------------------- a router's choice
@@ -425,5 +464,114 @@ extern "C" int lmsf_moe_route(const float* z, long z_stride, int n_tokens, int E
   hipLaunchKernelGGL(moe_route_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, stream, z, z_stride, n_tokens, E, top,
                      renorm, extra, choice, weight, gate);
   LMSF_LAUNCH_CHECK("moe_route");
+  return 0;
+}
+
+// The same with the scores a softmax over all experts (``softmax`` 1; 0: sigmoid) and a limit on where the choice may
+// fall: the experts form ``groups`` equal groups of neighbours, a group's score is its best expert's, and only experts
+// of the ``keep`` best groups can be chosen (groups = keep = 1: no limit). weight[n, k]: the chosen experts' scores
+// (over their sum with ``renorm``). A wave a token; a lane keeps the best score and the "kept" flag of the groups
+// lane, lane + 64, ... (at most 256 groups).
+__global__ __launch_bounds__(256) void moe_route_groups_kernel(const float* __restrict__ z, long z_stride, int n_tokens,
+                                                               int E, int top, int softmax, int groups, int keep,
+                                                               int renorm, int* __restrict__ choice,
+                                                               float* __restrict__ weight) {
+  const int n = blockIdx.x * (256 / LMSF_WAVE) + threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
+  if (n >= n_tokens) return;
+  const float* row = z + (long)n * z_stride;
+  float mx = -INFINITY, sum = 0.f;
+  if (softmax) {
+    for (int e = lane; e < E; e += LMSF_WAVE) mx = fmaxf(mx, row[e]);
+    mx = wave_max(mx);
+    for (int e = lane; e < E; e += LMSF_WAVE) sum += expf(row[e] - mx);
+    sum = wave_sum(sum);
+  }
+  const int per = E / groups;
+  float gbest[4];
+  unsigned kept = 0;           // bit i: group lane + 64 i is kept
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int g = lane + LMSF_WAVE * i;
+    gbest[i] = -INFINITY;
+    if (g < groups)
+      for (int e = g * per; e < (g + 1) * per; ++e) gbest[i] = fmaxf(gbest[i], row[e]);
+  }
+  if (keep >= groups) kept = 0xFu;
+  else
+    for (int k = 0; k < keep; ++k) {
+      float best = -INFINITY;
+      int best_g = groups;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int g = lane + LMSF_WAVE * i;
+        if (g < groups && !((kept >> i) & 1u) && (gbest[i] > best || (gbest[i] == best && g < best_g))) {
+          best = gbest[i];
+          best_g = g;
+        }
+      }
+#pragma unroll
+      for (int o = LMSF_WAVE / 2; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o, LMSF_WAVE);
+        const int og = __shfl_xor(best_g, o, LMSF_WAVE);
+        if (ob > best || (ob == best && og < best_g)) {
+          best = ob;
+          best_g = og;
+        }
+      }
+      if (best_g < groups && (best_g % LMSF_WAVE) == lane) kept |= 1u << (best_g / LMSF_WAVE);
+    }
+  float last = INFINITY, total = 0.f, mine = 0.f;
+  int last_e = -1, mine_e = 0;
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int best_e = E;
+    for (int e0 = 0; e0 < E; e0 += LMSF_WAVE) {      // (every lane takes part in the shuffle)
+      const int e = e0 + lane;
+      const int g = min(e, E - 1) / per;
+      const unsigned flags = __shfl(kept, g % LMSF_WAVE, LMSF_WAVE);
+      if (e >= E || !((flags >> (g / LMSF_WAVE)) & 1u)) continue;
+      const float sc = row[e];
+      const bool below = sc < last || (sc == last && e > last_e);
+      if (below && (sc > best || (sc == best && e < best_e))) {
+        best = sc;
+        best_e = e;
+      }
+    }
+#pragma unroll
+    for (int o = LMSF_WAVE / 2; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, LMSF_WAVE);
+      const int oe = __shfl_xor(best_e, o, LMSF_WAVE);
+      if (ob > best || (ob == best && oe < best_e)) {
+        best = ob;
+        best_e = oe;
+      }
+    }
+    last = best;
+    last_e = best_e;
+    const float sc = softmax ? expf(best - mx) / sum : 1.f / (1.f + expf(-best));
+    total += sc;
+    if (lane == k) {
+      mine = sc;
+      mine_e = min(best_e, E - 1);
+    }
+  }
+  if (lane < top) {
+    choice[(long)n * top + lane] = mine_e;
+    weight[(long)n * top + lane] = renorm ? mine / total : mine;
+  }
+}
+
+extern "C" int lmsf_moe_route_groups(const float* z, long z_stride, int n_tokens, int E, int top, int softmax,
+                                     int groups, int keep, int renorm, int* choice, float* weight,
+                                     hipStream_t stream) {
+  LMSF_CHECK(z && choice && weight, "moe_route_groups: null pointer");
+  LMSF_CHECK(E > 0 && top > 0 && top <= E && top <= LMSF_WAVE && z_stride >= E, "moe_route_groups: bad sizes");
+  LMSF_CHECK(groups > 0 && groups <= 256 && E % groups == 0 && keep > 0 && keep <= groups &&
+                 (long)keep * (E / groups) >= top,
+             "moe_route_groups: %d of %d groups of %d experts cannot hold %d choices", keep, groups, E, top);
+  if (n_tokens <= 0) return 0;
+  hipLaunchKernelGGL(moe_route_groups_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, stream, z, z_stride, n_tokens, E,
+                     top, softmax, groups, keep, renorm, choice, weight);
+  LMSF_LAUNCH_CHECK("moe_route_groups");
   return 0;
 }

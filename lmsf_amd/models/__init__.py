@@ -1,5 +1,5 @@
 """Architectures. Importing this package registers the built-in ones."""
-from . import llama, niresun, takosun, zevetar  # noqa: F401  (registration)
+from . import llama, murulorn, niresun, takosun, zevetar  # noqa: F401  (registration)
 from .decoder import DecoderModel
 
 __all__ = ["DecoderModel"]

@@ -76,6 +76,11 @@ class DecoderModel:
             out.append((m.cache_spec(), m.state_spec(), e.cache_from))
         return out
 
+    def embedding_state(self) -> Optional[StateSpec]:
+        """Per-request state that the embedding keeps (one tensor of the spec's shape per state slot), or None."""
+        spec = getattr(self.embedding, "state_spec", None)
+        return spec() if spec is not None else None
+
     def bind_cache(self, bindings: Sequence[CacheBinding]) -> None:
         if len(bindings) != len(self.schedule):
             raise ValueError("need one cache binding per schedule entry")
@@ -86,7 +91,10 @@ class DecoderModel:
     def forward(self, ctx, logits_out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Run the step's tokens; float32 logits [R, V] at ctx.logit_rows, in ``logits_out`` if one is given
         (a head that does not take ``out`` gets its result copied there)."""
-        residual = self.embedding.forward(ctx.token_ids)
+        if getattr(self.embedding, "needs_context", False):
+            residual = self.embedding.forward_step(ctx)        # an embedding that reads more of the step than the ids
+        else:
+            residual = self.embedding.forward(ctx.token_ids)
         branch = None
         for e, binding in zip(self.schedule, self.bindings):
             branch = self.blocks[e.layer].forward(branch, residual, ctx, binding)

@@ -436,12 +436,13 @@ class HipOps:
     def paged_attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                         block_tables: torch.Tensor, seg: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int, d: int,
                         scale: float, window: int = 0, batch=None, kernel: Optional[str] = None,
-                        chunk: int = 0, weights_f32: bool = False) -> torch.Tensor:
+                        chunk: int = 0, weights_f32: bool = False, softcap: float = 0.0) -> torch.Tensor:
         """Attention of every query token over the cached keys of its request: those at positions up to its own,
         within the last ``window`` positions if a window is given, or within its own chunk of ``chunk`` positions
         (chunks counted from position 0 of the request) if a chunk size is given. ``weights_f32``: in a bfloat16 run
         the softmax weights enter the product with the values in full float32 (as three bfloat16 parts on the
-        matrix cores) instead of rounded to bfloat16; scores, maxima and sums are float32 either way.
+        matrix cores) instead of rounded to bfloat16; scores, maxima and sums are float32 either way. ``softcap``
+        c > 0: a scaled score s enters the softmax as c tanh(s / c).
 
         ``q`` is [N, >= nh*d] with unit column stride (it may be the fused QKV buffer, of which the
         first nh*d columns are read). ``k_pages`` [pages, nkv, page_size, d], ``v_pages``
@@ -478,18 +479,18 @@ class HipOps:
             raise ValueError("the matrix-core attention kernels need bfloat16, a head size that is a multiple of 16 "
                              "up to 256, a page size that is a multiple of 4, 16-byte aligned query rows and a positive scale")
         if kernel == "generic" or not fast_ok:
-            self._check(self.lib.lmsf_paged_attention_generic(
+            self._check(self.lib.lmsf_paged_attention_generic_capped(
                 _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), num_pages,
                 _ptr(block_tables), block_tables.shape[1], _ptr(seg), _ptr(pos), N, nh, nkv, d, ps, float(scale),
-                int(window or 0), _code(q.dtype), self._stream()))
+                int(window or 0), float(softcap), _code(q.dtype), self._stream()))
             return out
         plan = self._attention_plan(batch, seg, pos, nh, nkv)
         exact = self.ATTENTION_WEIGHTS_F32 if weights_f32 else 0
         common = (_ptr(k_pages), _ptr(v_pages), num_pages, _ptr(block_tables), block_tables.shape[1])
         if plan.tiles is not None:
-            self._check(self.lib.lmsf_paged_attention_prefill_mfma(
+            self._check(self.lib.lmsf_paged_attention_prefill_mfma_capped(
                 _ptr(q), q.stride(0), _ptr(out), out.stride(0), *common, _ptr(plan.tiles), plan.n_tiles,
-                _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0),
+                _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0), float(softcap),
                 self.prefill_attention_variant + exact, self._stream()))
         if plan.n_single:
             c_chunk, c_splits = ctypes.c_int(0), ctypes.c_int(0)
@@ -498,10 +499,11 @@ class HipOps:
             chunk, n_splits = c_chunk.value, c_splits.value
             floats = self.lib.lmsf_attention_decode_scratch_floats(plan.n_single, nh, d, n_splits)
             scratch = torch.empty(floats if n_splits > 1 else 1, dtype=torch.float32, device=q.device)
-            self._check(self.lib.lmsf_paged_attention_decode_mfma(
+            self._check(self.lib.lmsf_paged_attention_decode_mfma_capped(
                 _ptr(q), q.stride(0), _ptr(out), out.stride(0), *common, _ptr(plan.single_tokens), plan.n_single,
                 None if plan.token_is_request else _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale),
-                int(window or 0), chunk, n_splits, _ptr(scratch), self.decode_attention_order + exact, self._stream()))
+                int(window or 0), float(softcap), chunk, n_splits, _ptr(scratch), self.decode_attention_order + exact,
+                self._stream()))
         return out
 
     ATTENTION_WEIGHTS_F32 = 256     # csrc/entry_points.h: LMSF_ATTENTION_WEIGHTS_F32
@@ -730,8 +732,11 @@ class HipOps:
 
     def table_moe(self, h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, token_ids: Optional[torch.Tensor],
                   table: torch.Tensor, weight: float, base: Optional[torch.Tensor] = None,
-                  pair_scale: Optional[torch.Tensor] = None, base_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  pair_scale: Optional[torch.Tensor] = None, base_scale: Optional[torch.Tensor] = None,
+                  out_scale: Optional[torch.Tensor] = None, gated: bool = True) -> torch.Tensor:
         """out[n] = base[n] + weight * sum_k down_e(silu(gate_e h[n]) * up_e h[n]) over e = table[token_ids[n], k].
+        ``gated`` False: experts of one matrix, ``w_gate_up`` [E, F, W], down_e(relu(up_e h[n])^2). ``out_scale``
+        (float32 [N, top]): what the expert of (n, k) returns is multiplied by out_scale[n, k].
         ``w_gate_up`` [E, 2 F, W] (gate rows first), ``w_down`` [E, W, F], ``table`` int32 [vocab, top].
         ``token_ids`` None: row n of the table is token n's choice (a router's, ``moe_route``). ``pair_scale``
         (float32 [N, top]): the expert of (n, k) gets pair_scale[n, k] * h[n] as its input. ``base_scale``
@@ -739,8 +744,8 @@ class HipOps:
         self._dev(h, w_gate_up, w_down, token_ids, table, base, pair_scale, base_scale)
         N, W = h.shape
         E, F2, _ = w_gate_up.shape
-        F = F2 // 2
-        if tuple(w_gate_up.shape) != (E, 2 * F, W) or tuple(w_down.shape) != (E, W, F) or not w_gate_up.is_contiguous() \
+        F = F2 // 2 if gated else F2
+        if tuple(w_gate_up.shape) != (E, (2 if gated else 1) * F, W) or tuple(w_down.shape) != (E, W, F) or not w_gate_up.is_contiguous() \
                 or not w_down.is_contiguous() or w_gate_up.dtype != h.dtype or w_down.dtype != h.dtype:
             raise ValueError("table_moe: expert weights must be contiguous [E, 2F, W] and [E, W, F] of h's dtype")
         if h.stride(1) != 1 or (base is not None and (base.shape != h.shape or base.stride(1) != 1 or base.dtype != h.dtype)):
@@ -757,6 +762,10 @@ class HipOps:
         if base_scale is not None and (base is None or base_scale.dtype != torch.float32 or base_scale.numel() != N
                                        or not base_scale.is_contiguous()):
             raise ValueError("table_moe: base_scale must be contiguous float32 [%d] beside a base" % N)
+        if out_scale is not None and (out_scale.dtype != torch.float32 or out_scale.numel() != N * top
+                                      or not out_scale.is_contiguous()):
+            raise ValueError("table_moe: out_scale must be contiguous float32 [%d, %d]" % (N, top))
+        self._dev(out_scale)
         act = torch.empty((N * top, F), dtype=h.dtype, device=h.device)
         out = torch.empty((N, W), dtype=h.dtype, device=h.device)
         ints = rows = None
@@ -764,11 +773,32 @@ class HipOps:
             # many tokens: grouped by expert on the device, tiles on the matrix cores
             ints = torch.empty(self.lib.lmsf_table_moe_scratch_ints(N, top, E), dtype=torch.int32, device=h.device)
             rows = torch.empty((N * top, W), dtype=torch.float32, device=h.device)
-        self._check(self.lib.lmsf_table_moe(
+        self._check(self.lib.lmsf_table_moe_act(
             _ptr(h), _code(h.dtype), h.stride(0), _ptr(w_gate_up), _ptr(w_down), _ptr(token_ids), _ptr(table), vocab,
             top, E, float(weight), _ptr(base), base.stride(0) if base is not None else 0, _ptr(pair_scale),
-            _ptr(base_scale), _ptr(act), _ptr(out), out.stride(0), N, F, W, _ptr(ints), _ptr(rows), self._stream()))
+            _ptr(base_scale), _ptr(out_scale), 0 if gated else 1, _ptr(act), _ptr(out), out.stride(0), N, F, W,
+            _ptr(ints), _ptr(rows), self._stream()))
         return out
+
+    def moe_route_groups(self, logits: torch.Tensor, experts: int, top: int, softmax: bool = True, groups: int = 1,
+                         keep: int = 1, renorm: bool = False):
+        """A router's choice from float32 logits [N, >= experts] with scores softmax(logits) over all experts (or
+        sigmoid), where only experts of the ``keep`` best of ``groups`` equal groups of neighbours may be chosen (a
+        group's score is its best expert's): (choice int32 [N, top], weight float32 [N, top]), the weights the
+        chosen experts' scores, over their sum with ``renorm``."""
+        self._dev(logits)
+        if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1 or logits.shape[1] < experts:
+            raise ValueError("moe_route_groups: logits must be float32 [N, >= %d] with unit column stride" % experts)
+        if not (0 < top <= experts and top <= 64) or not (0 < keep <= groups <= 256) or experts % groups \
+                or keep * (experts // groups) < top:
+            raise ValueError("moe_route_groups: %d of %d experts from %d of %d groups" % (top, experts, keep, groups))
+        N = logits.shape[0]
+        choice = torch.empty((N, top), dtype=torch.int32, device=logits.device)
+        weight = torch.empty((N, top), dtype=torch.float32, device=logits.device)
+        self._check(self.lib.lmsf_moe_route_groups(_ptr(logits), logits.stride(0), N, int(experts), int(top),
+                                                   1 if softmax else 0, int(groups), int(keep), 1 if renorm else 0,
+                                                   _ptr(choice), _ptr(weight), self._stream()))
+        return choice, weight
 
     def moe_route(self, logits: torch.Tensor, experts: int, top: int, renorm: bool = False, extra: int = -1):
         """A router's choice from float32 logits [N, >= experts]: (choice int32 [N, top], weight float32 [N, top],
@@ -788,6 +818,205 @@ class HipOps:
         self._check(self.lib.lmsf_moe_route(_ptr(logits), logits.stride(0), N, int(experts), int(top), 1 if renorm else 0,
                                             int(extra), _ptr(choice), _ptr(weight), _ptr(gate), self._stream()))
         return choice, weight, gate
+
+    # ------------------------------------------------------------------ what a token brings beside its embedding
+
+    def hashed_pair_embedding(self, batch, table: torch.Tensor, pairs: torch.Tensor, prev_state: torch.Tensor,
+                              mul_prev: int, mul_cur: int, keep: bool = False):
+        """float32 [N, W] = table[id] + pairs[(previous id * mul_prev + id * mul_cur) mod buckets], the last row of
+        ``pairs`` ([buckets + 1, W]) for a request's first token. The id before a segment's first token is
+        ``prev_state[slot]`` (int32, an entry per state slot and the spare one), which is brought up to date.
+        ``keep``: also returns a second copy of the result."""
+        ids = batch.token_ids
+        N = ids.numel()
+        self._dev(ids, table, pairs, prev_state, batch.positions)
+        if table.dim() != 2 or pairs.dim() != 2 or pairs.shape[1] != table.shape[1] or pairs.shape[0] < 2 \
+                or table.dtype != pairs.dtype or not table.is_contiguous() or not pairs.is_contiguous():
+            raise ValueError("hashed_pair_embedding: table [V, W] and pairs [buckets + 1, W] of one dtype are needed")
+        if prev_state.dtype != torch.int32 or not prev_state.is_contiguous():
+            raise ValueError("hashed_pair_embedding: prev_state must be contiguous int32")
+        self._i32(ids, "token_ids", N)
+        self._i32(batch.positions, "positions", N)
+        seg_of, seg_starts, slots, S = self._segments(batch, N)
+        V, W = table.shape
+        out = torch.empty((N, W), dtype=torch.float32, device=table.device)
+        kept = torch.empty((N, W), dtype=torch.float32, device=table.device) if keep else None
+        self._check(self.lib.lmsf_hashed_pair_embedding(
+            _ptr(ids), _ptr(batch.positions), _ptr(seg_of), _ptr(seg_starts), _ptr(slots), _ptr(prev_state), _ptr(table),
+            _ptr(pairs), _code(table.dtype), _ptr(out), _ptr(kept), N, S, V, W, pairs.shape[0] - 1, int(mul_prev),
+            int(mul_cur), self._stream()))
+        return (out, kept) if keep else out
+
+    def concat_rows(self, a: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        """[a | b] row by row in ``out_dtype``; a, b contiguous float32 [N, Wa], [N, Wb]."""
+        self._dev(a, b)
+        if a.dim() != 2 or b.dim() != 2 or a.shape[0] != b.shape[0] or a.dtype != torch.float32 \
+                or b.dtype != torch.float32 or not a.is_contiguous() or not b.is_contiguous():
+            raise ValueError("concat_rows: two contiguous float32 matrices of equal rows are needed")
+        out = torch.empty((a.shape[0], a.shape[1] + b.shape[1]), dtype=out_dtype, device=a.device)
+        self._check(self.lib.lmsf_concat_rows(_ptr(a), _ptr(b), _ptr(out), _code(out_dtype), a.shape[0], a.shape[1],
+                                              b.shape[1], self._stream()))
+        return out
+
+    def gate_table(self, z: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, at: int) -> torch.Tensor:
+        """gelu_tanh(z [N, dim]) * table[ids, at : at + dim], in z's dtype."""
+        self._dev(z, ids, table)
+        N, dim = z.shape
+        if z.stride(1) != 1 or table.dim() != 2 or table.dtype != z.dtype or table.stride(1) != 1 \
+                or not (0 <= at and at + dim <= table.shape[1]):
+            raise ValueError("gate_table: z [N, dim] and a table [V, >= at + dim] of one dtype are needed")
+        self._i32(ids, "token_ids", N)
+        out = torch.empty((N, dim), dtype=z.dtype, device=z.device)
+        self._check(self.lib.lmsf_gate_table(_ptr(z), z.stride(0), _ptr(ids), _ptr(table), table.stride(0), int(at),
+                                             table.shape[0], _ptr(out), _code(z.dtype), N, dim, self._stream()))
+        return out
+
+    def relu_squared(self, z: torch.Tensor) -> torch.Tensor:
+        """relu(z)^2, elementwise, in z's dtype; z [N, F] with unit column stride."""
+        self._dev(z)
+        if z.dim() != 2 or z.stride(1) != 1:
+            raise ValueError("relu_squared: z must be [N, F] with unit column stride")
+        out = torch.empty(tuple(z.shape), dtype=z.dtype, device=z.device)
+        self._check(self.lib.lmsf_relu_squared(_ptr(z), z.stride(0), _ptr(out), _code(z.dtype), z.shape[0], z.shape[1],
+                                               self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ attention with norms and rotated values
+
+    def attn_prepare_normed(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, kv_heads: int, dim: int,
+                            vdim: int, padded: int, positions: torch.Tensor, slots: Optional[torch.Tensor],
+                            k_pages: torch.Tensor, v_pages: torch.Tensor, q_weight: Optional[torch.Tensor] = None,
+                            k_weight: Optional[torch.Tensor] = None, eps: float = 1e-5,
+                            table: Optional[torch.Tensor] = None, table_v: Optional[torch.Tensor] = None,
+                            interleaved: bool = False, v_norm: bool = False) -> torch.Tensor:
+        """Readies projected queries, keys and values for ``paged_attention`` at head size ``padded``, each step
+        optional: one RMS norm over all of q with ``q_weight`` (float32 [heads * dim]) and one over all of k with
+        ``k_weight``; rotation of the first table.shape[1] entries of every q and k head; every value head over its
+        root mean square (``v_norm``); rotation of all of a value head (``table_v`` float32 [max_pos, vdim]). Pairs
+        are (2m, 2m + 1) if ``interleaved`` else (m, m + rot / 2). k and v go to the tokens' slots of the pages.
+        Returns q [N, heads * padded]."""
+        self._dev(q, k, v, positions, slots, k_pages, v_pages, q_weight, k_weight, table, table_v)
+        N = q.shape[0]
+        for t, w, name in ((q, heads * dim, "q"), (k, kv_heads * dim, "k"), (v, kv_heads * vdim, "v")):
+            if t.dim() != 2 or t.shape[0] != N or t.shape[1] < w or t.stride(1) != 1 or t.dtype != q.dtype:
+                raise ValueError("attn_prepare_normed: %s must be [%d, >= %d] of q's dtype with unit column stride"
+                                 % (name, N, w))
+        self._i32(positions, "positions", N)
+        self._i32(slots, "slots", N)
+        if q_weight is not None:
+            self._f32_vec(q_weight, heads * dim, "attn_prepare_normed: q_weight")
+        if k_weight is not None:
+            self._f32_vec(k_weight, kv_heads * dim, "attn_prepare_normed: k_weight")
+        rot = 0
+        max_pos = None
+        for tb, width, name in ((table, None, "table"), (table_v, vdim, "table_v")):
+            if tb is None:
+                continue
+            if tb.dtype != torch.float32 or tb.dim() != 2 or not tb.is_contiguous() or tb.shape[1] % 2 \
+                    or (width is not None and tb.shape[1] != width) or (width is None and tb.shape[1] > dim) \
+                    or (max_pos is not None and tb.shape[0] != max_pos):
+                raise ValueError("attn_prepare_normed: %s must be contiguous float32 [max_pos, entries]" % name)
+            max_pos = tb.shape[0]
+        if table is not None:
+            rot = table.shape[1]
+        if k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != padded or not k_pages.is_contiguous() \
+                or k_pages.dtype != q.dtype:
+            raise ValueError("attn_prepare_normed: k_pages must be contiguous [pages, %d, page_size, %d] of %s"
+                             % (kv_heads, padded, q.dtype))
+        num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+        if tuple(v_pages.shape) != (num_pages, kv_heads, padded, ps) or not v_pages.is_contiguous() or v_pages.dtype != q.dtype:
+            raise ValueError("attn_prepare_normed: v_pages must be contiguous [%d, %d, %d, %d] of %s"
+                             % (num_pages, kv_heads, padded, ps, q.dtype))
+        out = torch.empty((N, heads * padded), dtype=q.dtype, device=q.device)
+        self._check(self.lib.lmsf_attn_prepare_normed(
+            _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _code(q.dtype), _ptr(q_weight),
+            _ptr(k_weight), float(eps), _ptr(positions), _ptr(table), rot, _ptr(table_v), int(max_pos or 1),
+            1 if interleaved else 0, 1 if v_norm else 0, _ptr(slots), _ptr(out), out.stride(0), _ptr(k_pages),
+            _ptr(v_pages), num_pages, N, int(heads), int(kv_heads), int(dim), int(vdim), int(padded), ps, self._stream()))
+        return out
+
+    def attn_finish(self, a: torch.Tensor, padded: int, heads: int, vdim: int, positions: torch.Tensor,
+                    gate: Optional[torch.Tensor] = None, table_v: Optional[torch.Tensor] = None,
+                    interleaved: bool = False) -> torch.Tensor:
+        """The attention's result [N, heads * padded] made ready for the output projection: every head's first vdim
+        entries, turned back by the token's position over all of them (``table_v`` float32 [max_pos, vdim]; None: not),
+        times sigmoid(gate[n, h]) (``gate`` [N, >= heads], one number a head; None: none). Returns [N, heads * vdim]."""
+        self._dev(a, positions, gate, table_v)
+        N = a.shape[0]
+        if a.dim() != 2 or a.stride(1) != 1 or a.shape[1] < heads * padded or padded < vdim:
+            raise ValueError("attn_finish: a must be [N, >= %d] with unit column stride" % (heads * padded))
+        self._i32(positions, "positions", N)
+        if gate is not None and (gate.dim() != 2 or gate.shape[0] != N or gate.shape[1] < heads or gate.stride(1) != 1
+                                 or gate.dtype != a.dtype):
+            raise ValueError("attn_finish: gate must be [%d, >= %d] of a's dtype" % (N, heads))
+        if table_v is not None and (table_v.dtype != torch.float32 or table_v.dim() != 2 or table_v.shape[1] != vdim
+                                    or not table_v.is_contiguous()):
+            raise ValueError("attn_finish: table_v must be contiguous float32 [max_pos, %d]" % vdim)
+        out = torch.empty((N, heads * vdim), dtype=a.dtype, device=a.device)
+        self._check(self.lib.lmsf_attn_finish(
+            _ptr(a), a.stride(0), _ptr(gate), gate.stride(0) if gate is not None else 0, _code(a.dtype), _ptr(positions),
+            _ptr(table_v), table_v.shape[0] if table_v is not None else 1, 1 if interleaved else 0, _ptr(out),
+            out.stride(0), N, int(heads), int(vdim), int(padded), self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ the gated delta rule
+
+    def gated_delta_state_floats(self, heads: int, dim: int, vdim: int) -> int:
+        return int(self.lib.lmsf_gated_delta_state_floats(heads, dim, vdim))
+
+    def gated_delta(self, qkv: torch.Tensor, q_at: int, k_at: int, v_at: int, a: torch.Tensor, dt_bias: torch.Tensor,
+                    a_log: torch.Tensor, b: torch.Tensor, state: torch.Tensor, batch, heads: int, kv_heads: int,
+                    dim: int, vdim: int, q_scale: float, unit_eps: float = 1e-6) -> torch.Tensor:
+        """The gated delta rule over each request's tokens, the memory S [heads, dim, vdim] carried in ``state``
+        (float32 [slots, >= heads * dim * vdim]): S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, with
+        q, k the unit vectors of columns q_at, k_at of ``qkv`` (kv_heads heads of dim; q times q_scale), v its columns
+        from v_at (heads of vdim), beta = sigmoid(b [N, >= heads]) and g = exp(-exp(a_log [heads]) softplus(a + dt_bias))
+        (``a`` float32 [N, heads * dim]). Returns the heads' o as float32 [N, heads * vdim]."""
+        self._dev(qkv, a, dt_bias, a_log, b)
+        N = qkv.shape[0]
+        need = max(q_at + kv_heads * dim, k_at + kv_heads * dim, v_at + heads * vdim)
+        if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < need:
+            raise ValueError("gated_delta: qkv must be [N, >= %d] with unit column stride" % need)
+        if a.dtype != torch.float32 or a.dim() != 2 or a.shape[0] != N or a.shape[1] < heads * dim or a.stride(1) != 1:
+            raise ValueError("gated_delta: a must be float32 [%d, >= %d]" % (N, heads * dim))
+        if b.dtype != torch.float32 or b.dim() != 2 or b.shape[0] != N or b.shape[1] < heads or b.stride(1) != 1:
+            raise ValueError("gated_delta: b must be float32 [%d, >= %d]" % (N, heads))
+        self._f32_vec(dt_bias, heads * dim, "gated_delta: dt_bias")
+        self._f32_vec(a_log, heads, "gated_delta: a_log")
+        if heads % kv_heads or dim > 256:
+            raise ValueError("gated_delta: %d heads over %d key heads, keys of %d entries (at most 256)" % (heads, kv_heads, dim))
+        self._state_view(state, self.gated_delta_state_floats(heads, dim, vdim), "gated_delta")
+        _, seg_starts, slots, S = self._segments(batch, N)
+        out = torch.empty((N, heads * vdim), dtype=torch.float32, device=qkv.device)
+        self._check(self.lib.lmsf_gated_delta(
+            _ptr(qkv), _code(qkv.dtype), qkv.stride(0), int(q_at), int(k_at), int(v_at), _ptr(a), a.stride(0),
+            _ptr(dt_bias), _ptr(a_log), _ptr(b), b.stride(0), _ptr(state), state.stride(0), _ptr(seg_starts), _ptr(slots),
+            _ptr(out), out.stride(0), N, S, int(heads), int(kv_heads), int(dim), int(vdim), float(q_scale),
+            float(unit_eps), self._stream()))
+        return out
+
+    def head_rms_gate(self, raw: torch.Tensor, heads: int, vdim: int, eps: float, weight: Optional[torch.Tensor],
+                      gate: Optional[torch.Tensor], out_dtype: torch.dtype, activation: str = "sigmoid") -> torch.Tensor:
+        """Every head of ``raw`` (float32 [N, heads * vdim]) over its root mean square, times ``weight`` (float32
+        [vdim], shared by the heads; None: none), times sigmoid or silu of ``gate`` ([N, >= heads * vdim] of
+        ``out_dtype``; None: none). Returns [N, heads * vdim] in ``out_dtype``."""
+        self._dev(raw, weight, gate)
+        N = raw.shape[0]
+        if raw.dtype != torch.float32 or raw.dim() != 2 or raw.shape[1] < heads * vdim or raw.stride(1) != 1:
+            raise ValueError("head_rms_gate: raw must be float32 [N, >= %d]" % (heads * vdim))
+        if weight is not None:
+            self._f32_vec(weight, vdim, "head_rms_gate: weight")
+        act = 0
+        if gate is not None:
+            if gate.dim() != 2 or gate.shape[0] != N or gate.shape[1] < heads * vdim or gate.stride(1) != 1 \
+                    or gate.dtype != out_dtype:
+                raise ValueError("head_rms_gate: gate must be [%d, >= %d] of the output's dtype" % (N, heads * vdim))
+            act = {"sigmoid": 1, "silu": 2}[activation]
+        out = torch.empty((N, heads * vdim), dtype=out_dtype, device=raw.device)
+        self._check(self.lib.lmsf_head_rms_gate(
+            _ptr(raw), raw.stride(0), _ptr(weight), _ptr(gate), gate.stride(0) if gate is not None else 0, act, _ptr(out),
+            out.stride(0), _code(out_dtype), N, int(heads), int(vdim), float(eps), self._stream()))
+        return out
 
     # ------------------------------------------------------------------ layer scale, logit cap
 

@@ -10,7 +10,7 @@ from typing import Optional
 from ..csrc import build as _build
 from .dispatch import ProductShape, Route, Tunables
 
-ABI_VERSION = 29
+ABI_VERSION = 30
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -39,6 +39,31 @@ _SIGNATURES = {
     "lmsf_paged_attention_decode_mfma": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, _P, c_int, _P, c_int, _P, _P,
                                                  c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P, c_int,
                                                  _P]),
+    "lmsf_paged_attention_generic_capped": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, _P, c_int, _P, _P, c_int,
+                                                    c_int, c_int, c_int, c_int, c_float, c_int, c_float, c_int, _P]),
+    "lmsf_paged_attention_prefill_mfma_capped": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, _P, c_int, _P, c_int, _P,
+                                                         _P, c_int, c_int, c_int, c_int, c_float, c_int, c_float, c_int,
+                                                         _P]),
+    "lmsf_paged_attention_decode_mfma_capped": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, _P, c_int, _P, c_int, _P,
+                                                        _P, c_int, c_int, c_int, c_int, c_float, c_int, c_float, c_int,
+                                                        c_int, _P, c_int, _P]),
+    "lmsf_hashed_pair_embedding": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int,
+                                           c_int, c_long, c_long, _P]),
+    "lmsf_concat_rows": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, _P]),
+    "lmsf_gate_table": (c_int, [_P, c_long, _P, _P, c_long, c_int, c_int, _P, c_int, c_int, c_int, _P]),
+    "lmsf_relu_squared": (c_int, [_P, c_long, _P, c_int, c_int, c_int, _P]),
+    "lmsf_attn_prepare_normed": (c_int, [_P, c_long, _P, c_long, _P, c_long, c_int, _P, _P, c_float, _P, _P, c_int, _P,
+                                         c_int, c_int, c_int, _P, _P, c_long, _P, _P, c_long, c_int, c_int, c_int, c_int,
+                                         c_int, c_int, c_int, _P]),
+    "lmsf_attn_finish": (c_int, [_P, c_long, _P, c_long, c_int, _P, _P, c_int, c_int, _P, c_long, c_int, c_int, c_int,
+                                 c_int, _P]),
+    "lmsf_gated_delta_state_floats": (c_long, [c_int, c_int, c_int]),
+    "lmsf_gated_delta": (c_int, [_P, c_int, c_long, c_int, c_int, c_int, _P, c_long, _P, _P, _P, c_long, _P, c_long, _P,
+                                 _P, _P, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, _P]),
+    "lmsf_head_rms_gate": (c_int, [_P, c_long, _P, _P, c_long, c_int, _P, c_long, c_int, c_int, c_int, c_int, c_float, _P]),
+    "lmsf_table_moe_act": (c_int, [_P, c_int, c_long, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, c_long, _P, _P, _P,
+                                   c_int, _P, _P, c_long, c_int, c_int, c_int, _P, _P, _P]),
+    "lmsf_moe_route_groups": (c_int, [_P, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, _P]),
     "lmsf_group_norm": (c_int, [_P, c_int, c_long, _P, _P, _P, c_long, c_int, _P, _P, _P, c_int, c_long, _P, c_int, c_int,
                                 c_int, c_float, c_float, _P]),
     "lmsf_latent_cache_write": (c_int, [_P, c_int, c_long, _P, c_float, _P, _P, c_int, c_int, _P, _P, _P, c_long, c_int,

@@ -2,8 +2,9 @@
 from .base import (Block, CacheBinding, CacheSpec, FeedForward, LayerSpec, Mixer, ModelSpec, Norm, Part,
                    PartSpec, PositionEncoding, Runtime, ScheduleEntry, StateSpec, TensorDecl, build_part,
                    part_class, register_part, unregister_part)
-from . import (attention, block, dyt_norm, embedding, flex_attention, group_norm, latent_attention,  # noqa: F401  (registration)
-               mlp, norm, parallel, recurrent, retention, rotary, routed_moe, table_moe)
+from . import (attention, block, delta_rule, dyt_norm, embedding, flex_attention, group_norm,  # noqa: F401  (registration)
+               latent_attention, mlp, norm, normed_attention, parallel, recurrent, retention, rotary, routed_moe,
+               table_moe)
 from .linear import FusedLinear, Linear
 
 __all__ = ["Block", "CacheBinding", "CacheSpec", "FeedForward", "LayerSpec", "Mixer", "ModelSpec", "Norm", "Part",

@@ -3,7 +3,8 @@ from typing import Optional
 
 import torch
 
-from .base import Block, CacheBinding, Runtime, build_part, register_part
+from .base import Block, CacheBinding, Part, Runtime, TensorDecl, build_part, register_part
+from .linear import Linear
 
 
 @register_part("block", "prenorm_residual")
@@ -196,4 +197,120 @@ class ParallelScaledBlock(Block):
                                            eps=nxt.eps if nxt is not None else 0.0)
         if ahead is not None:
             ctx.aux["prenormed"] = ahead
+        return None
+
+
+class StreamInjection(Part):
+    """x <- M [x ; x0]: the stream and the embedding's output side by side through one matrix [W, 2 W] (the stream's
+    columns first). The product's operands are in the run's type, its result and the stream float32."""
+
+    graph_safe = True
+    recordable = False
+
+    def __init__(self, name: str, rt: Runtime, hidden_size: int):
+        super().__init__(name, rt)
+        self.W = int(hidden_size)
+        self.proj = Linear("", rt, name, 2 * self.W, self.W, bare_names=True)
+
+    def children(self):
+        return [self.proj]
+
+    def forward(self, residual: torch.Tensor, ctx) -> None:
+        x0 = ctx.aux.get("embedding_output")
+        if x0 is None:
+            raise ValueError("%s: the embedding did not keep its output for this step" % self.prefix)
+        ops = self.rt.ops
+        both = ops.concat_rows(residual, x0, self.rt.dtype)
+        residual.copy_(ops.linear_wide(both, self.proj.weight, None))
+
+
+class TokenSideInput(Part):
+    """A per-layer input from the token itself, added to the stream: e = a slice of the token's row of a table shared
+    by the layers; g = gelu_tanh(W_gate x) * e; y = W_proj g; x += y / rms(y) * w (a plain RMS-norm weight)."""
+
+    graph_safe = True
+    recordable = False
+
+    def __init__(self, prefix: str, rt: Runtime, hidden_size: int, dim: int, at: int, table_name: str, table_width: int,
+                 vocab_size: int, eps: float, gate_name: str = "gate", proj_name: str = "proj", norm_name: str = "norm"):
+        super().__init__(prefix, rt)
+        self.W, self.dim, self.at, self.eps = int(hidden_size), int(dim), int(at), float(eps)
+        self.table_name, self.table_shape = str(table_name), (int(vocab_size), int(table_width))
+        if not (0 <= self.at and self.at + self.dim <= self.table_shape[1]):
+            raise ValueError("%s: entries %d to %d of a table row of %d" % (prefix, at, at + dim, table_width))
+        self.gate = Linear(prefix, rt, gate_name, self.W, self.dim, bare_names=True)
+        self.proj = Linear(prefix, rt, proj_name, self.dim, self.W, bare_names=True)
+        self.norm_name = "%s.%s" % (prefix, norm_name)
+        self.table: Optional[torch.Tensor] = None
+        self.norm_weight: Optional[torch.Tensor] = None
+
+    def children(self):
+        return [self.gate, self.proj]
+
+    def checkpoint_tensors(self):
+        return {self.table_name: TensorDecl(self.table_shape),
+                self.norm_name: TensorDecl((self.W,), init="ones", keeps_float32=True)}
+
+    def load_weights(self, fetch) -> None:
+        self.table = fetch(self.table_name).contiguous()            # (one device tensor for all layers: the loader shares it)
+        self.norm_weight = fetch(self.norm_name).to(torch.float32).contiguous()
+
+    def tensors(self):
+        return [t for t in (self.norm_weight,) if t is not None]
+
+    def forward(self, residual: torch.Tensor, ctx) -> None:
+        ops = self.rt.ops
+        x = ops.group_norm(residual=residual, out_dtype=self.rt.dtype)          # the stream in the run's type
+        g = ops.gate_table(self.gate.forward(x), ctx.token_ids, self.table, self.at)
+        y = ops.linear_wide(g, self.proj.weight, None)
+        ops.group_norm(x=y, x_weight=self.norm_weight, residual=residual, x_eps=self.eps, want_out=False)
+
+
+@register_part("block", "sandwich")
+class SandwichBlock(Block):
+    """A norm before and after each sublayer:
+
+        x += norm_b(mixer(norm_a(x)));   x += norm_d(ffn(norm_c(x)))
+
+    (without a feed-forward only the first), optionally with the stream replaced by a product over the stream and the
+    embedding's output before the block (``inject``: the name of the matrix; a block that begins a pass of a loop over
+    layers) and a per-layer input from the token added after it (``side``: the parameters of ``TokenSideInput``). The
+    stream is float32; nothing is left to add when the block returns. The addition after the mixer and the norm
+    before the feed-forward are one kernel. The reference's only arrangement is the pre-norm one
+    (core/src/model_executor/models/llama/llama.rs:286-340)."""
+
+    graph_safe = True
+    recordable = False
+
+    ROLES = ("pre_mixer", "post_mixer")          # "pre_ffn" and "post_ffn" too where there is a feed-forward
+
+    def __init__(self, prefix: str, rt: Runtime, mixer, feed_forward, norms, hidden_size: int,
+                 inject: Optional[str] = None, side=None):
+        super().__init__(prefix, rt, mixer, feed_forward, norms)
+        self.has_ffn = not getattr(feed_forward, "absent", False)
+        if self.has_ffn and not ("pre_ffn" in norms and "post_ffn" in norms):
+            raise ValueError("block %s needs the norms pre_ffn and post_ffn around its feed-forward" % prefix)
+        self.inject = StreamInjection(inject, rt, hidden_size) if inject else None
+        self.side = TokenSideInput("%s.%s" % (prefix, dict(side).pop("prefix", "side")), rt, hidden_size=hidden_size,
+                                   **{k: v for k, v in dict(side).items() if k != "prefix"}) if side else None
+        self._ffn_takes_ids = bool(getattr(feed_forward, "needs_token_ids", False))
+
+    def children(self):
+        return super().children() + [p for p in (self.inject, self.side) if p is not None]
+
+    def forward(self, branch: Optional[torch.Tensor], residual: torch.Tensor, ctx, binding: CacheBinding):
+        if branch is not None:
+            raise ValueError("sandwich takes no branch that is still to be added")
+        n = self.norms
+        if self.inject is not None:
+            self.inject.forward(residual, ctx)
+        a = self.mixer.forward(n["pre_mixer"].forward(residual), ctx, binding)
+        if self.has_ffn:
+            h = n["post_mixer"].add_normed(a, residual, then=n["pre_ffn"])
+            f = self.feed_forward.forward(h, token_ids=ctx.token_ids) if self._ffn_takes_ids else self.feed_forward.forward(h)
+            n["post_ffn"].add_normed(f, residual)
+        else:
+            n["post_mixer"].add_normed(a, residual)
+        if self.side is not None:
+            self.side.forward(residual, ctx)
         return None

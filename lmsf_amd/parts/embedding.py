@@ -10,7 +10,7 @@ from typing import Callable, Dict, Optional
 
 import torch
 
-from .base import Part, Runtime, TensorDecl, register_part
+from .base import Part, Runtime, StateSpec, TensorDecl, register_part
 
 
 @register_part("embedding", "token_embedding")
@@ -34,6 +34,64 @@ class TokenEmbedding(Part):
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         """int32 [N] -> float32 [N, H]."""
         return self.rt.ops.embedding(token_ids, self.weight, self.scale)
+
+
+@register_part("embedding", "hashed_pair_embedding")
+class HashedPairEmbedding(Part):
+    """x = table[id] + pairs[row]: beside the token's own row a row of a second table chosen by a hash of the token
+    before it and the token, row = (previous id * mul_prev + id * mul_cur) mod buckets; a request's first token takes
+    the table's last row (number ``buckets``). The sum is float32. The token before a step's first token is part of
+    the request's state: one int32 per state slot (``state_spec``; the engine hands the tensor over through
+    ``bind_state``), written by the kernel that reads it. ``keep_output``: the result is also left in
+    ``ctx.aux["embedding_output"]`` for parts that read it after the stream has moved on. The reference's embedding is
+    the plain row gather (core/src/model_executor/layers/vocab_parallel_embedding.rs:28-38)."""
+
+    graph_safe = True
+    recordable = False
+    needs_context = True            # the model calls forward_step(ctx) instead of forward(token_ids)
+
+    def __init__(self, prefix: str, rt: Runtime, vocab_size: int, hidden_size: int, buckets: int, mul_prev: int,
+                 mul_cur: int, pair_name: str = "bigram", weight_name: str = "", keep_output: bool = False):
+        super().__init__(prefix, rt)
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
+        if self.buckets < 1 or self.mul_prev < 0 or self.mul_cur < 0:
+            raise ValueError("hashed_pair_embedding: buckets must be > 0 and the multipliers >= 0")
+        self.weight_name = "%s.%s" % (prefix, weight_name) if weight_name else prefix
+        self.pair_name = str(pair_name)
+        self.keep_output = bool(keep_output)
+        self.weight: Optional[torch.Tensor] = None
+        self.pairs: Optional[torch.Tensor] = None
+        self.prev_state: Optional[torch.Tensor] = None
+
+    def checkpoint_tensors(self) -> Dict[str, TensorDecl]:
+        return {self.weight_name: TensorDecl((self.vocab_size, self.hidden_size)),
+                self.pair_name: TensorDecl((self.buckets + 1, self.hidden_size))}
+
+    def load_weights(self, fetch: Callable[[str], torch.Tensor]) -> None:
+        self.weight = fetch(self.weight_name).contiguous()
+        self.pairs = fetch(self.pair_name).to(self.weight.dtype).contiguous()
+
+    def tensors(self):
+        return [t for t in (self.weight, self.pairs) if t is not None]
+
+    def state_spec(self) -> StateSpec:
+        return StateSpec((1,), torch.int32)
+
+    def bind_state(self, state: torch.Tensor) -> None:
+        self.prev_state = state.view(-1)
+
+    def forward_step(self, ctx) -> torch.Tensor:
+        """The step's tokens -> float32 [N, H]."""
+        if self.prev_state is None:
+            raise ValueError("hashed_pair_embedding: no state was bound (the token before a step's first)")
+        if not self.keep_output:
+            return self.rt.ops.hashed_pair_embedding(ctx, self.weight, self.pairs, self.prev_state, self.mul_prev,
+                                                     self.mul_cur)
+        x, kept = self.rt.ops.hashed_pair_embedding(ctx, self.weight, self.pairs, self.prev_state, self.mul_prev,
+                                                    self.mul_cur, keep=True)
+        ctx.aux["embedding_output"] = kept
+        return x
 
 
 @register_part("head", "lm_head")

@@ -14,24 +14,29 @@ from .base import Norm, Part, Runtime, TensorDecl, register_part
 
 @register_part("norm", "group_rms_norm")
 class GroupRMSNorm(Norm):
-    """``weight_name`` is appended to the prefix with a dot ("" : the tensor is the prefix itself)."""
+    """``weight_name`` is appended to the prefix with a dot ("" : the tensor is the prefix itself). ``weight_offset``
+    is added to the stored weight at load (1 for a weight that is stored around zero and acts as 1 + w)."""
 
     graph_safe = True
     recordable = False
 
-    def __init__(self, prefix: str, rt: Runtime, size: int, eps: float, groups: int = 1, weight_name: str = "weight"):
+    def __init__(self, prefix: str, rt: Runtime, size: int, eps: float, groups: int = 1, weight_name: str = "weight",
+                 weight_offset: float = 0.0):
         super().__init__(prefix, rt)
         self.size, self.eps, self.groups = int(size), float(eps), int(groups)
+        self.weight_offset = float(weight_offset)
         if self.groups <= 0 or self.size % self.groups:
             raise ValueError("norm %r: %d columns do not split into %d groups" % (prefix, self.size, self.groups))
         self.weight_name = "%s.%s" % (prefix, weight_name) if weight_name else prefix
         self.weight: Optional[torch.Tensor] = None
 
     def checkpoint_tensors(self) -> Dict[str, TensorDecl]:
-        return {self.weight_name: TensorDecl((self.size,), init="ones", keeps_float32=True)}
+        init = "ones" if self.weight_offset == 0.0 else "zeros"
+        return {self.weight_name: TensorDecl((self.size,), init=init, keeps_float32=True)}
 
     def load_weights(self, fetch: Callable[[str], torch.Tensor]) -> None:
-        self.weight = fetch(self.weight_name).to(torch.float32).contiguous()
+        w = fetch(self.weight_name).to(torch.float32)
+        self.weight = (w + self.weight_offset if self.weight_offset != 0.0 else w).contiguous()
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """gn of a float32 stream (or of activations, also a view with unit column stride) in the run's dtype."""

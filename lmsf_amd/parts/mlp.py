@@ -34,3 +34,26 @@ class GatedMLP(FeedForward):
     def forward(self, h: torch.Tensor, pending_ok: bool = False):
         a = self.rt.ops.linear_gated(h, self.gate_up.weight, self.gate_up.bias, self.activation)
         return self.down.forward(a, pending_ok=pending_ok)
+
+
+@register_part("feed_forward", "plain_mlp")
+class PlainMLP(FeedForward):
+    """y = W_down act(W_up x), one matrix in and one out; act is the square of relu. The reference's feed-forward is the
+    gated one above."""
+
+    graph_safe = True
+    recordable = False
+
+    def __init__(self, prefix: str, rt: Runtime, hidden_size: int, intermediate_size: int,
+                 activation: str = "relu_squared", up_name: str = "up", down_name: str = "down", bare_names: bool = True):
+        super().__init__(prefix, rt)
+        if activation != "relu_squared":
+            raise ValueError("plain_mlp activation %r unknown (relu_squared)" % activation)
+        self.up = Linear(prefix, rt, up_name, hidden_size, intermediate_size, bare_names=bare_names)
+        self.down = Linear(prefix, rt, down_name, intermediate_size, hidden_size, bare_names=bare_names)
+
+    def children(self):
+        return [self.up, self.down]
+
+    def forward(self, h: torch.Tensor):
+        return self.down.forward(self.rt.ops.relu_squared(self.up.forward(h)))

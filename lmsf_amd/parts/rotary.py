@@ -71,8 +71,13 @@ class RotaryEncoding(PositionEncoding):
     graph_safe = True
 
     def __init__(self, prefix: str, rt: Runtime, head_dim: int, theta: float, rotary_dim: Optional[int] = None,
-                 scaling: Optional[Mapping[str, Any]] = None, style: str = "neox"):
+                 scaling: Optional[Mapping[str, Any]] = None, style: str = "neox", angles: str = "float32"):
         super().__init__(prefix, rt)
+        # "float64": frequencies, angles, cosines and sines are worked out in float64 and rounded once, into the
+        # float32 table (unscaled frequencies only); "float32": in float32 throughout, as the reference does
+        if angles not in ("float32", "float64") or (angles == "float64" and scaling):
+            raise ValueError("rotary angles %r unknown (float32, float64 without scaling)" % angles)
+        self.angles = angles
         self.head_dim = int(head_dim)
         self.rotary_dim = int(rotary_dim) if rotary_dim else self.head_dim
         if self.rotary_dim % 2 or self.rotary_dim > self.head_dim or self.rotary_dim <= 0:
@@ -86,10 +91,16 @@ class RotaryEncoding(PositionEncoding):
 
     def _key(self):
         sc = None if self.scaling is None else tuple(sorted(self.scaling.items()))
-        return ("rotary_table", self.rotary_dim, self.theta, sc, self.rt.max_positions)
+        return ("rotary_table", self.rotary_dim, self.theta, sc, self.rt.max_positions, self.angles)
 
     def load_weights(self, fetch: Callable[[str], torch.Tensor]) -> None:
         key = self._key()
+        if key not in self.rt.shared and self.angles == "float64":
+            idx = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
+            inv = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * idx / self.rotary_dim)
+            angles = torch.arange(self.rt.max_positions, dtype=torch.float64)[:, None] * inv[None, :]
+            table = torch.cat([torch.cos(angles), torch.sin(angles)], dim=1).to(torch.float32).contiguous()
+            self.rt.shared[key] = table.to(self.rt.device)
         if key not in self.rt.shared:
             inv = inverse_frequencies(self.rotary_dim, self.theta, self.scaling)
             pos = torch.arange(self.rt.max_positions, dtype=torch.float32)

@@ -125,7 +125,7 @@ class TorchOps:
 
     # ------------------------------------------------------------ attention
     def paged_attention(self, q, k_pages, v_pages, block_tables, seg, pos, nh, nkv, d, scale, window=0, batch=None,
-                        kernel=None, chunk=0, weights_f32=False):
+                        kernel=None, chunk=0, weights_f32=False, softcap=0.0):
         N = q.shape[0]
         ps = k_pages.shape[2]
         out = torch.empty((N, nh * d), dtype=q.dtype, device=q.device)
@@ -143,6 +143,8 @@ class TorchOps:
             keys = keys.repeat_interleave(rep, dim=1)                    # [n, nh, d]
             vals = vals.repeat_interleave(rep, dim=1)
             sc = torch.einsum("hd,nhd->hn", qt, keys) * scale
+            if softcap and softcap > 0:
+                sc = softcap * torch.tanh(sc / softcap)
             pr = torch.softmax(sc, dim=-1)
             out[t] = torch.einsum("hn,nhd->hd", pr, vals).reshape(nh * d).to(q.dtype)
         return out
@@ -220,15 +222,19 @@ class TorchOps:
             out[:, h * out_head + out_at:h * out_head + out_at + width] = self._rotate(v, cs, table.shape[1]).to(out.dtype)
             out[:, h * out_head + out_at + width:(h + 1) * out_head] = 0
 
-    def table_moe(self, h, w_gate_up, w_down, token_ids, table, weight, base=None, pair_scale=None, base_scale=None):
-        F = w_gate_up.shape[1] // 2
+    def table_moe(self, h, w_gate_up, w_down, token_ids, table, weight, base=None, pair_scale=None, base_scale=None,
+                  out_scale=None, gated=True):
+        F = w_gate_up.shape[1] // 2 if gated else w_gate_up.shape[1]
         out = torch.zeros(h.shape, dtype=torch.float32)
         for n in range(h.shape[0]):
             for k, e in enumerate(table[int(token_ids[n]) if token_ids is not None else n].tolist()):
                 x = h[n].to(torch.float32) * (float(pair_scale[n, k]) if pair_scale is not None else 1.0)
                 gu = (w_gate_up[e].to(torch.float32) @ x).to(h.dtype).to(torch.float32)
-                a = (gu[:F] / (1.0 + torch.exp(-gu[:F])) * gu[F:]).to(h.dtype).to(torch.float32)
-                out[n] += w_down[e].to(torch.float32) @ a
+                if gated:
+                    a = (gu[:F] / (1.0 + torch.exp(-gu[:F])) * gu[F:]).to(h.dtype).to(torch.float32)
+                else:
+                    a = (torch.relu(gu) ** 2).to(h.dtype).to(torch.float32)
+                out[n] += (w_down[e].to(torch.float32) @ a) * (float(out_scale[n, k]) if out_scale is not None else 1.0)
         out = out * weight
         if base is not None:
             b = base.to(torch.float32)
@@ -244,6 +250,147 @@ class TorchOps:
             w = w / w.sum(-1, keepdim=True)
         gate = torch.sigmoid(logits[:, extra]).contiguous() if extra >= 0 else None
         return order.to(torch.int32).contiguous(), w.contiguous(), gate
+
+    # ------------------------------------------------------------ a token's extras, norms and rotated values, delta rule
+    def moe_route_groups(self, logits, experts, top, softmax=True, groups=1, keep=1, renorm=False):
+        z = logits[:, :experts].to(torch.float32)
+        sc = torch.softmax(z, -1) if softmax else torch.sigmoid(z)
+        N = z.shape[0]
+        per = experts // groups
+        best = z.reshape(N, groups, per).max(-1).values
+        kept = torch.zeros((N, groups), dtype=torch.bool)
+        kept.scatter_(1, torch.topk(best, keep, -1).indices, True)
+        masked = z.masked_fill(~kept.repeat_interleave(per, 1), float("-inf"))
+        choice = torch.topk(masked, top, -1).indices
+        w = torch.gather(sc, 1, choice)
+        if renorm:
+            w = w / w.sum(-1, keepdim=True)
+        return choice.to(torch.int32), w.contiguous()
+
+    def hashed_pair_embedding(self, batch, table, pairs, prev_state, mul_prev, mul_cur, keep=False):
+        ids = batch.token_ids.long()
+        buckets = pairs.shape[0] - 1
+        rows = torch.empty_like(ids)
+        for t0, t1, slot in self._segments(batch):
+            for t in range(t0, t1):
+                if int(batch.positions[t]) == 0:
+                    rows[t] = buckets
+                    continue
+                prev = int(prev_state[slot]) if t == t0 else int(ids[t - 1])
+                rows[t] = (prev * int(mul_prev) + int(ids[t]) * int(mul_cur)) % buckets
+            if t1 > t0:
+                prev_state[slot] = int(ids[t1 - 1])
+        out = table[ids].to(torch.float32) + pairs[rows].to(torch.float32)
+        return (out, out.clone()) if keep else out
+
+    def concat_rows(self, a, b, out_dtype):
+        return torch.cat([a, b], -1).to(out_dtype)
+
+    def gate_table(self, z, ids, table, at):
+        zf = z.to(torch.float32)
+        g = 0.5 * zf * (1.0 + torch.tanh(0.7978845608028654 * (zf + 0.044715 * zf ** 3)))
+        return (g * table[ids.long()][:, at:at + z.shape[1]].to(torch.float32)).to(z.dtype)
+
+    def relu_squared(self, z):
+        return (torch.relu(z.to(torch.float32)) ** 2).to(z.dtype)
+
+    @staticmethod
+    def _turn(x, cs, interleaved, sign=1.0):
+        """x [..., n] turned in pairs by the angles of cs [..., n] = [cos | sin] (broadcast over heads)."""
+        n = cs.shape[-1]
+        c, s = cs[..., :n // 2], cs[..., n // 2:] * sign
+        out = x.clone()
+        if interleaved:
+            a, b = x[..., 0:n:2], x[..., 1:n:2]
+            out[..., 0:n:2] = a * c - b * s
+            out[..., 1:n:2] = b * c + a * s
+        else:
+            a, b = x[..., :n // 2], x[..., n // 2:n]
+            out[..., :n // 2] = a * c - b * s
+            out[..., n // 2:n] = b * c + a * s
+        return out
+
+    def attn_prepare_normed(self, q, k, v, heads, kv_heads, dim, vdim, padded, positions, slots, k_pages, v_pages,
+                            q_weight=None, k_weight=None, eps=1e-5, table=None, table_v=None, interleaved=False,
+                            v_norm=False):
+        N = q.shape[0]
+        qf = q[:, :heads * dim].to(torch.float32)
+        kf = k[:, :kv_heads * dim].to(torch.float32)
+        vf = v[:, :kv_heads * vdim].to(torch.float32).reshape(N, kv_heads, vdim)
+        if q_weight is not None:
+            qf = qf / torch.sqrt((qf * qf).mean(-1, keepdim=True) + eps) * q_weight
+        if k_weight is not None:
+            kf = kf / torch.sqrt((kf * kf).mean(-1, keepdim=True) + eps) * k_weight
+        qf, kf = qf.reshape(N, heads, dim), kf.reshape(N, kv_heads, dim)
+        if table is not None:
+            rot = table.shape[1]
+            cs = table[positions.long()][:, None, :]
+            qf = torch.cat([self._turn(qf[..., :rot], cs, interleaved), qf[..., rot:]], -1)
+            kf = torch.cat([self._turn(kf[..., :rot], cs, interleaved), kf[..., rot:]], -1)
+        if v_norm:
+            vf = vf / torch.sqrt((vf * vf).mean(-1, keepdim=True) + eps)
+        if table_v is not None:
+            vf = self._turn(vf, table_v[positions.long()][:, None, :], interleaved)
+        out = torch.zeros((N, heads, padded), dtype=q.dtype)
+        out[..., :dim] = qf.to(q.dtype)
+        if slots is not None:
+            ps = k_pages.shape[2]
+            sl = slots.long()
+            ok = sl >= 0
+            page, off = sl[ok] // ps, sl[ok] % ps
+            kp = torch.zeros((N, kv_heads, padded), dtype=q.dtype)
+            kp[..., :dim] = kf.to(q.dtype)
+            vp = torch.zeros((N, kv_heads, padded), dtype=q.dtype)
+            vp[..., :vdim] = vf.to(q.dtype)
+            k_pages[page, :, off, :] = kp[ok]
+            v_pages[page, :, :, off] = vp[ok]
+        return out.reshape(N, heads * padded)
+
+    def attn_finish(self, a, padded, heads, vdim, positions, gate=None, table_v=None, interleaved=False):
+        N = a.shape[0]
+        x = a[:, :heads * padded].to(torch.float32).reshape(N, heads, padded)[..., :vdim]
+        if table_v is not None:
+            x = self._turn(x, table_v[positions.long()][:, None, :], interleaved, sign=-1.0)
+        if gate is not None:
+            x = x * torch.sigmoid(gate[:, :heads].to(torch.float32))[:, :, None]
+        return x.reshape(N, heads * vdim).to(a.dtype)
+
+    def gated_delta_state_floats(self, heads, dim, vdim):
+        return heads * dim * vdim
+
+    def gated_delta(self, qkv, q_at, k_at, v_at, a, dt_bias, a_log, b, state, batch, heads, kv_heads, dim, vdim,
+                    q_scale, unit_eps=1e-6):
+        N = qkv.shape[0]
+        rep = heads // kv_heads
+        q = qkv[:, q_at:q_at + kv_heads * dim].to(torch.float32).reshape(N, kv_heads, dim)
+        k = qkv[:, k_at:k_at + kv_heads * dim].to(torch.float32).reshape(N, kv_heads, dim)
+        v = qkv[:, v_at:v_at + heads * vdim].to(torch.float32).reshape(N, heads, vdim)
+        q = (q / torch.sqrt((q * q).sum(-1, keepdim=True) + unit_eps) * q_scale).repeat_interleave(rep, 1)
+        k = (k / torch.sqrt((k * k).sum(-1, keepdim=True) + unit_eps)).repeat_interleave(rep, 1)
+        beta = torch.sigmoid(b[:, :heads])
+        g = torch.exp(-torch.exp(a_log)[None, :, None] * torch.nn.functional.softplus(
+            a[:, :heads * dim] + dt_bias).reshape(N, heads, dim))
+        out = torch.zeros((N, heads, vdim), dtype=torch.float32)
+        for t0, t1, slot in self._segments(batch):
+            S = state[slot, :heads * dim * vdim].reshape(heads, dim, vdim).clone()
+            for t in range(t0, t1):
+                S = S * g[t][:, :, None]
+                u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k[t]))
+                S = S + k[t][:, :, None] * u[:, None, :]
+                out[t] = torch.einsum("hdv,hd->hv", S, q[t])
+            state[slot, :heads * dim * vdim] = S.reshape(-1)
+        return out.reshape(N, heads * vdim)
+
+    def head_rms_gate(self, raw, heads, vdim, eps, weight, gate, out_dtype, activation="sigmoid"):
+        N = raw.shape[0]
+        x = raw[:, :heads * vdim].reshape(N, heads, vdim)
+        y = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+        if weight is not None:
+            y = y * weight
+        if gate is not None:
+            g = gate[:, :heads * vdim].to(torch.float32).reshape(N, heads, vdim)
+            y = y * (torch.sigmoid(g) if activation == "sigmoid" else g * torch.sigmoid(g))
+        return y.reshape(N, heads * vdim).to(out_dtype)
 
     def scale_add_norm(self, a, scale_a, b, scale_b, residual, weight=None, eps=1e-5):
         r = residual + scale_a * a.to(torch.float32)
