@@ -489,6 +489,37 @@ def zevetar_shapes(name):
     return zev, tako
 
 
+def murulorn_shapes(name):
+    """A Murulorn configuration at sizes that resemble a real model's layers, and beside it the Zevetar configuration
+    of equal width and number of layer runs (the closest architecture of the package: attention within a window, a
+    matrix memory per head, routed experts). Murulorn has six layers of which the second and third run twice: eight
+    runs going attention + dense, (attention + experts, delta rule + experts) twice, delta rule + dense, attention +
+    dense, delta rule + experts; keys and values of 128 entries in 16 heads over 4, a window of 1,024; a memory of 16
+    heads of 64 x 128 as Zevetar's retention has."""
+    zev, _ = zevetar_shapes(name)
+    W = zev["width"]
+    H, ff, E, eff = {"2b": (16, 8192, 16, 1024), "7b": (32, 14336, 32, 2048)}[name]
+    att = {"heads": H, "kv_heads": H // 4, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
+           "rot": {"base": 1e6, "dims": 64}, "mask": {"size": 1024}}
+    mem = {"heads": H, "kv_heads": H, "dim": 64, "vdim": 128, "conv": 4, "decay_rank": 64, "gate_rank": 64}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": E, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    kinds = [("attention", att, dense), ("attention", att, moe), ("channel_delta", mem, moe), ("channel_delta", mem, dense),
+             ("attention", att, dense), ("channel_delta", mem, moe)]
+    layers = [{"type": t, "mixer": dict(m), "mlp": dict(f)} for t, m, f in kinds]
+    mur = {"architecture": "Murulorn", "vocab": zev["vocab"], "width": W, "norm": {"eps": 1e-6},
+           "embedding": {"bigram": {"buckets": 100003, "mul_prev": 1000003, "mul_cur": 31}}, "token_side": {"dim": 64},
+           "loop": {"start": 1, "stop": 3, "times": 2}, "layers": layers, "max_position_embeddings": 8192,
+           "torch_dtype": "bfloat16"}
+    return mur, zev
+
+
+def murulorn_run(args):
+    """``--workload murulorn``: prefill and decode of a Murulorn model beside the Zevetar model of equal width and layer
+    runs; one JSON line, as for the other designs."""
+    beside_llama_run(args, "murulorn", args.murulorn_sizes, murulorn_shapes(args.murulorn_sizes), twin="zevetar")
+
+
 def takosun_run(args):
     """``--workload takosun``: prefill and decode of a Takosun model beside the Llama model of equal size; one JSON
     line. Decode: ``--steps`` steps at batch 1, 8 and 64 after 512-token prompts; prefill: one request of 512 and of
@@ -556,17 +587,20 @@ def main():
     ap.add_argument("--max-num-batched-tokens", type=int, default=8192)
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.85)
     ap.add_argument("--skip-points", action="store_true", help="leave out the batch 1 and batch 64 runs")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "products", "takosun", "niresun", "zevetar"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "products", "takosun", "niresun", "zevetar", "murulorn"],
                     help="decode: the default line (Llama-3-8B shape); serve: continuous batching of 64 requests at "
                          "Llama-2-7B shape, a line of its own; products: a layer's matrix products alone, the "
                          "library's against the engine's choice, at --rows; takosun: a Takosun model beside the Llama model "
                          "of equal size, prefill and decode; niresun: the same for a Niresun model; zevetar: a Zevetar "
-                         "model beside the Takosun model of equal size")
+                         "model beside the Takosun model of equal size; murulorn: a Murulorn model beside the Zevetar "
+                         "model of equal width and layer runs")
     ap.add_argument("--takosun-sizes", default="2b", choices=["2b", "7b"], help="takosun: the layers' sizes")
     ap.add_argument("--niresun-sizes", default="2b", choices=["2b", "7b"],
                     help="niresun: the layers' sizes (a Niresun model beside the Llama model of equal size)")
     ap.add_argument("--zevetar-sizes", default="2b", choices=["2b", "7b"],
                     help="zevetar: the layers' sizes (a Zevetar model beside the Takosun model of equal size)")
+    ap.add_argument("--murulorn-sizes", default="2b", choices=["2b", "7b"],
+                    help="murulorn: the layers' sizes (a Murulorn model beside the Zevetar model of equal width and layer runs)")
     ap.add_argument("--rows", default="17,64,100,128,129,192,256,512,2048", help="products: numbers of rows")
     ap.add_argument("--prefill-chunk-size", type=int, default=1024, help="serve: longest portion of a prompt in a step")
     ap.add_argument("--shape", default="llama3-8b", choices=sorted(SHAPES),
@@ -607,6 +641,9 @@ def main():
         return
     if args.workload == "niresun":
         niresun_run(args)
+        return
+    if args.workload == "murulorn":
+        murulorn_run(args)
         return
     if args.workload == "zevetar":
         zevetar_run(args)
