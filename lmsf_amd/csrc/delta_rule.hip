@@ -8,159 +8,224 @@
 // rows of S. H value heads and G query/key heads (head h reads q/k head h / (H / G)). S lives in the request's state
 // slot, float32 [H, dim, vdim], and is read once and written once a step.
 //
-// The columns of S are independent of one another: column j only ever needs k, q, g, beta and v_j. A wave holds 16
-// columns, each spread over four lanes that keep a quarter of its rows each in registers (RPL rows a
-// lane; dim is padded to 4 RPL with rows whose k and q are zero), and two shuffles add the four partial dot
-// products; a workgroup of four waves shares what it makes of k, q and g for eight tokens at a time in LDS. Tokens of
-// a request run one after the other; (request, head, 64 columns) side by side. A step of single tokens is the same
-// kernel with one token a workgroup, bound by the memory's bytes: S in and out.
+// The columns of S are independent of one another: column j only ever needs k, q, g, beta and v_j, and a token's step
+// is a chain of dependent operations over the rows of a column, so what bounds a long segment is the time of one
+// step, not the chip's rate. Hence two kernels. The first makes k, q and g of every (token, head) ready, side by side
+// for all tokens: unit vectors, decays, beta, written as float32 in the order in which the second reads them. The
+// second runs the recurrence with a column's rows spread over 16 lanes (RPL = rows a lane holds, in registers; the
+// key size is padded to 16 RPL with rows whose k and q are zero), four columns a wave, a wave a workgroup: a step is
+// RPL multiplications and 3 RPL multiply-adds a lane and two reductions over 16 lanes, and the operands of the next
+// tokens are asked for while the present ones are worked on (they do not depend on S). Tokens of a request run one
+// after the other; (request, head, 4 columns) side by side: 512 waves for 16 heads of 128 columns. The state lies as
+// [H, ceil(vdim / 4), dim, 4], so that a wave's part of it is one piece of memory; a step of single tokens is the same
+// kernels, bound by the memory's bytes: S in and out.
 //
-// A second kernel divides every head's o by its root mean square, multiplies by a weight over vdim (shared by the
+// A third kernel divides every head's o by its root mean square, multiplies by a weight over vdim (shared by the
 // heads) and by sigmoid or silu of a gate, and rounds to the run's type.
 #include "common.h"
 
 #include <math.h>
 
-#define DELTA_TB 8            // tokens made ready at a time
-#define DELTA_COLS 64         // value columns a workgroup holds
+#define DELTA_R 16            // lanes that share a column
+#define DELTA_CPW 4           // columns a wave holds
 
 __device__ __forceinline__ float softplus_f32(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
-template <typename T, int RPL>
-__global__ __launch_bounds__(256) void gated_delta_kernel(
-    const T* __restrict__ qkv, long stride, int q_at, int k_at, int v_at, const float* __restrict__ a, long a_stride,
+static inline int delta_rows_per_lane(int dim) { return dim <= 16 ? 1 : dim <= 32 ? 2 : dim <= 64 ? 4 : dim <= 128 ? 8 : 16; }
+
+// prep [N, H, 3, DP] float32: k, q, g of every (token, head), entry p = r * RPL + ii holding row ii * 16 + r;
+// beta_out [N, H]. A wave a (token, head).
+template <typename T>
+__global__ __launch_bounds__(256) void gated_delta_prepare_kernel(
+    const T* __restrict__ qkv, long stride, int q_at, int k_at, const float* __restrict__ a, long a_stride,
     const float* __restrict__ dt_bias, const float* __restrict__ a_log, const float* __restrict__ b, long b_stride,
-    float* __restrict__ state, long state_stride, const int* __restrict__ seg_starts, const int* __restrict__ slots,
-    float* __restrict__ out, long out_stride, int H, int G, int dim, int vdim, float q_scale, float unit_eps) {
-  constexpr int PAD = RPL == 8 ? 0 : 8;
-  constexpr int LD = 4 * (RPL + PAD);             // floats of one staged vector
-  __shared__ __attribute__((aligned(16))) float sk[DELTA_TB][LD], sq[DELTA_TB][LD], sg[DELTA_TB][LD];
-  __shared__ float sv[DELTA_TB][DELTA_COLS], sbeta[DELTA_TB];
-  const int s = blockIdx.x, h = blockIdx.y, c0 = blockIdx.z * DELTA_COLS;
-  const int tid = threadIdx.x, wave = tid / LMSF_WAVE, lane = tid % LMSF_WAVE;
-  const int r = lane / 16, col = c0 + wave * 16 + lane % 16;
-  const bool col_ok = col < vdim;
-  const int t0 = seg_starts[s], t1 = seg_starts[s + 1];
-  if (t1 <= t0) return;
-  const int gh = h / (H / G);
-  float* S = state + (long)slots[s] * state_stride + (long)h * dim * vdim;
-  float st[RPL];
-#pragma unroll
-  for (int ii = 0; ii < RPL; ++ii) {
-    const int i = r * RPL + ii;
-    st[ii] = (col_ok && i < dim) ? S[(long)i * vdim + col] : 0.f;
+    float* __restrict__ prep, float* __restrict__ beta_out, int n_tokens, int H, int G, int dim, int RPL, float q_scale,
+    float unit_eps) {
+  const long w = (long)blockIdx.x * (256 / LMSF_WAVE) + threadIdx.x / LMSF_WAVE;
+  const int lane = threadIdx.x % LMSF_WAVE;
+  if (w >= (long)n_tokens * H) return;
+  const long t = w / H;
+  const int h = (int)(w - t * H), gh = h / (H / G), DP = DELTA_R * RPL;
+  const T* qr = qkv + t * stride + q_at + gh * dim;
+  const T* kr = qkv + t * stride + k_at + gh * dim;
+  float ssq = 0.f, ssk = 0.f;
+  for (int i = lane; i < dim; i += LMSF_WAVE) {
+    const float x = to_f32<T>(qr[i]), y = to_f32<T>(kr[i]);
+    ssq += x * x;
+    ssk += y * y;
   }
-  const float decay_rate = expf(a_log[h]);
-  const int dim_pad = 4 * RPL;
-  for (int tb = t0; tb < t1; tb += DELTA_TB) {
-    const int nt = min(DELTA_TB, t1 - tb);
-    __syncthreads();                                // the batch before has been read
-    // 32 threads a token: unit vectors, decays
-    {
-      const int j = tid / 32, l = tid % 32;
-      if (j < nt) {
-        const long t = tb + j;
-        const T* qr = qkv + t * stride + q_at + gh * dim;
-        const T* kr = qkv + t * stride + k_at + gh * dim;
-        float ssq = 0.f, ssk = 0.f;
-        for (int i = l; i < dim; i += 32) {
-          const float x = to_f32<T>(qr[i]), y = to_f32<T>(kr[i]);
-          ssq += x * x;
-          ssk += y * y;
-        }
-#pragma unroll
-        for (int o = 16; o > 0; o >>= 1) {
-          ssq += __shfl_xor(ssq, o, LMSF_WAVE);
-          ssk += __shfl_xor(ssk, o, LMSF_WAVE);
-        }
-        const float iq = q_scale / sqrtf(ssq + unit_eps), ik = 1.f / sqrtf(ssk + unit_eps);
-        for (int i = l; i < dim_pad; i += 32) {
-          const int at = (i / RPL) * (RPL + PAD) + i % RPL;
-          float kq = 0.f, kk = 0.f, g = 1.f;
-          if (i < dim) {
-            kq = to_f32<T>(qr[i]) * iq;
-            kk = to_f32<T>(kr[i]) * ik;
-            g = expf(-decay_rate * softplus_f32(a[t * a_stride + h * dim + i] + dt_bias[h * dim + i]));
-          }
-          sq[j][at] = kq;
-          sk[j][at] = kk;
-          sg[j][at] = g;
-        }
-        if (l == 0) sbeta[j] = 1.f / (1.f + expf(-b[t * b_stride + h]));
-      }
-      for (int e = tid; e < nt * DELTA_COLS; e += 256) {
-        const int jj = e / DELTA_COLS, c = e % DELTA_COLS;
-        sv[jj][c] = c0 + c < vdim ? to_f32<T>(qkv[(long)(tb + jj) * stride + v_at + h * vdim + c0 + c]) : 0.f;
-      }
+  const float iq = q_scale / sqrtf(wave_sum(ssq) + unit_eps), ik = 1.f / sqrtf(wave_sum(ssk) + unit_eps);
+  const float rate = expf(a_log[h]);
+  float* out = prep + w * 3 * DP;
+  for (int p = lane; p < DP; p += LMSF_WAVE) {
+    const int i = (p % RPL) * DELTA_R + p / RPL;
+    float kk = 0.f, kq = 0.f, g = 1.f;
+    if (i < dim) {
+      kk = to_f32<T>(kr[i]) * ik;
+      kq = to_f32<T>(qr[i]) * iq;
+      g = expf(-rate * softplus_f32(a[t * a_stride + h * dim + i] + dt_bias[h * dim + i]));
     }
-    __syncthreads();
-    for (int j = 0; j < nt; ++j) {
-      const float* pk = &sk[j][r * (RPL + PAD)];
-      const float* pq = &sq[j][r * (RPL + PAD)];
-      const float* pg = &sg[j][r * (RPL + PAD)];
-      float dot = 0.f;
-#pragma unroll
-      for (int ii = 0; ii < RPL; ++ii) {
-        st[ii] *= pg[ii];
-        dot = fmaf(pk[ii], st[ii], dot);
-      }
-      dot += __shfl_xor(dot, 16, LMSF_WAVE);
-      dot += __shfl_xor(dot, 32, LMSF_WAVE);
-      const float u = sbeta[j] * (sv[j][wave * 16 + lane % 16] - dot);
-      float o = 0.f;
-#pragma unroll
-      for (int ii = 0; ii < RPL; ++ii) {
-        st[ii] = fmaf(pk[ii], u, st[ii]);
-        o = fmaf(pq[ii], st[ii], o);
-      }
-      o += __shfl_xor(o, 16, LMSF_WAVE);
-      o += __shfl_xor(o, 32, LMSF_WAVE);
-      if (r == 0 && col_ok) out[(long)(tb + j) * out_stride + h * vdim + col] = o;
-    }
+    out[p] = kk;
+    out[DP + p] = kq;
+    out[2 * DP + p] = g;
   }
+  if (lane == 0) beta_out[w] = 1.f / (1.f + expf(-b[t * b_stride + h]));
+}
+
+template <int RPL>
+struct DeltaToken {
+  float k[RPL], q[RPL], g[RPL], beta, v;
+};
+
+template <int RPL>
+__device__ __forceinline__ void delta_load_vec(float* dst, const float* __restrict__ src) {
+  if constexpr (RPL >= 4) {
 #pragma unroll
-  for (int ii = 0; ii < RPL; ++ii) {
-    const int i = r * RPL + ii;
-    if (col_ok && i < dim) S[(long)i * vdim + col] = st[ii];
+    for (int j = 0; j < RPL / 4; ++j) {
+      const float4 x = *reinterpret_cast<const float4*>(src + 4 * j);
+      dst[4 * j] = x.x; dst[4 * j + 1] = x.y; dst[4 * j + 2] = x.z; dst[4 * j + 3] = x.w;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < RPL; ++j) dst[j] = src[j];
   }
 }
 
-extern "C" long lmsf_gated_delta_state_floats(int H, int dim, int vdim) { return (long)H * dim * vdim; }
+__device__ __forceinline__ float delta_sum16(float v) {
+  v += __shfl_xor(v, 8, LMSF_WAVE);
+  v += __shfl_xor(v, 4, LMSF_WAVE);
+  v += __shfl_xor(v, 2, LMSF_WAVE);
+  v += __shfl_xor(v, 1, LMSF_WAVE);
+  return v;
+}
+
+template <typename T, int RPL>
+__global__ __launch_bounds__(LMSF_WAVE) void gated_delta_recurrence_kernel(
+    const T* __restrict__ qkv, long stride, int v_at, const float* __restrict__ prep, const float* __restrict__ beta,
+    float* __restrict__ state, long state_stride, const int* __restrict__ seg_starts, const int* __restrict__ slots,
+    float* __restrict__ out, long out_stride, int H, int dim, int vdim) {
+  constexpr int DP = DELTA_R * RPL;
+  constexpr int U = RPL >= 8 ? 2 : 4;              // tokens whose operands are in registers ahead of their turn
+  const int s = blockIdx.x, h = blockIdx.y, cb = blockIdx.z;
+  const int lane = threadIdx.x, c = lane / DELTA_R, r = lane % DELTA_R;
+  const int col = cb * DELTA_CPW + c;
+  const bool col_ok = col < vdim;
+  const int t0 = seg_starts[s], t1 = seg_starts[s + 1];
+  if (t1 <= t0) return;
+  const int n_cb = (vdim + DELTA_CPW - 1) / DELTA_CPW;
+  float* S = state + (long)slots[s] * state_stride + ((long)h * n_cb + cb) * dim * DELTA_CPW;
+  float st[RPL];
+#pragma unroll
+  for (int ii = 0; ii < RPL; ++ii) {
+    const int i = ii * DELTA_R + r;
+    st[ii] = i < dim ? S[i * DELTA_CPW + c] : 0.f;
+  }
+  auto fetch = [&](DeltaToken<RPL>& tk, int t) {
+    t = min(t, t1 - 1);                            // (beyond the segment: the last token again, not used)
+    const float* base = prep + ((long)t * H + h) * 3 * DP + r * RPL;
+    delta_load_vec<RPL>(tk.k, base);
+    delta_load_vec<RPL>(tk.q, base + DP);
+    delta_load_vec<RPL>(tk.g, base + 2 * DP);
+    tk.beta = beta[(long)t * H + h];
+    tk.v = col_ok ? to_f32<T>(qkv[(long)t * stride + v_at + h * vdim + col]) : 0.f;
+  };
+  DeltaToken<RPL> cur[U], nxt[U];
+#pragma unroll
+  for (int j = 0; j < U; ++j) fetch(cur[j], t0 + j);
+  for (int tb = t0; tb < t1; tb += U) {
+    if (tb + U < t1) {
+#pragma unroll
+      for (int j = 0; j < U; ++j) fetch(nxt[j], tb + U + j);
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) {
+      if (tb + j < t1) {
+        const DeltaToken<RPL>& tk = cur[j];
+        float dot = 0.f;
+#pragma unroll
+        for (int ii = 0; ii < RPL; ++ii) {
+          st[ii] *= tk.g[ii];
+          dot = fmaf(tk.k[ii], st[ii], dot);
+        }
+        dot = delta_sum16(dot);
+        const float u = tk.beta * (tk.v - dot);
+        float o = 0.f;
+#pragma unroll
+        for (int ii = 0; ii < RPL; ++ii) {
+          st[ii] = fmaf(tk.k[ii], u, st[ii]);
+          o = fmaf(tk.q[ii], st[ii], o);
+        }
+        o = delta_sum16(o);
+        if (r == 0 && col_ok) out[(long)(tb + j) * out_stride + h * vdim + col] = o;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < U; ++j) cur[j] = nxt[j];
+  }
+#pragma unroll
+  for (int ii = 0; ii < RPL; ++ii) {
+    const int i = ii * DELTA_R + r;
+    if (i < dim) S[i * DELTA_CPW + c] = st[ii];
+  }
+}
+
+// floats of a request's memory: [H, ceil(vdim / 4), dim, 4]
+extern "C" long lmsf_gated_delta_state_floats(int H, int dim, int vdim) {
+  return (long)H * ((vdim + DELTA_CPW - 1) / DELTA_CPW) * dim * DELTA_CPW;
+}
+
+// floats of scratch for n_tokens tokens: what the first kernel hands the second
+extern "C" long lmsf_gated_delta_scratch_floats(int n_tokens, int H, int dim) {
+  return (long)n_tokens * H * (3 * DELTA_R * delta_rows_per_lane(dim) + 1);
+}
 
 // qkv: the (convolved, activated) q [N, G dim], k [N, G dim], v [N, H vdim] as columns q_at, k_at, v_at of one buffer
 // of ``dtype`` with row stride ``stride``; a: float32 [N, H dim] before bias and softplus; dt_bias float32 [H dim];
-// a_log float32 [H]; b: float32 [N, >= H] before the sigmoid; state float32 [slots, >= H dim vdim]; out: float32
-// [N, H vdim], the heads' read-outs as they are.
+// a_log float32 [H]; b: float32 [N, >= H] before the sigmoid; state float32 [slots, >= lmsf_gated_delta_state_floats];
+// scratch: lmsf_gated_delta_scratch_floats floats, 16-byte aligned; out: float32 [N, H vdim], the heads' read-outs as
+// they are.
 extern "C" int lmsf_gated_delta(const void* qkv, int dtype, long stride, int q_at, int k_at, int v_at, const float* a,
                                 long a_stride, const float* dt_bias, const float* a_log, const float* b,
                                 long b_stride, float* state, long state_stride, const int* seg_starts,
-                                const int* slots, float* out, long out_stride, int n_tokens, int n_segments, int H,
-                                int G, int dim, int vdim, float q_scale, float unit_eps, hipStream_t stream) {
-  LMSF_CHECK(qkv && a && dt_bias && a_log && b && state && seg_starts && slots && out, "gated_delta: null pointer");
+                                const int* slots, float* scratch, float* out, long out_stride, int n_tokens,
+                                int n_segments, int H, int G, int dim, int vdim, float q_scale, float unit_eps,
+                                hipStream_t stream) {
+  LMSF_CHECK(qkv && a && dt_bias && a_log && b && state && seg_starts && slots && out && scratch,
+             "gated_delta: null pointer");
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "gated_delta: unknown dtype code %d", dtype);
   LMSF_CHECK(H > 0 && G > 0 && H % G == 0 && dim > 0 && dim <= 256 && vdim > 0,
              "gated_delta: heads %d over %d key heads, keys of %d (at most 256) and values of %d entries", H, G, dim, vdim);
-  LMSF_CHECK(H <= 65535 && (vdim + DELTA_COLS - 1) / DELTA_COLS <= 65535, "gated_delta: too many heads or columns");
+  const int n_cb = (vdim + DELTA_CPW - 1) / DELTA_CPW;
+  LMSF_CHECK(H <= 65535 && n_cb <= 65535, "gated_delta: too many heads or columns");
   LMSF_CHECK(a_stride >= (long)H * dim && b_stride >= H && out_stride >= (long)H * vdim &&
-                 state_stride >= (long)H * dim * vdim && q_at >= 0 && k_at >= 0 && v_at >= 0,
+                 state_stride >= lmsf_gated_delta_state_floats(H, dim, vdim) && q_at >= 0 && k_at >= 0 && v_at >= 0,
              "gated_delta: strides too small");
+  LMSF_CHECK(lmsf_aligned16(scratch), "gated_delta: the scratch must be 16-byte aligned");
   if (n_tokens <= 0 || n_segments <= 0) return 0;
-  const dim3 grid(n_segments, H, (vdim + DELTA_COLS - 1) / DELTA_COLS);
-#define DELTA_LAUNCH(T, R)                                                                                          \
-  hipLaunchKernelGGL((gated_delta_kernel<T, R>), grid, dim3(256), 0, stream, (const T*)qkv, stride, q_at, k_at, v_at, \
-                     a, a_stride, dt_bias, a_log, b, b_stride, state, state_stride, seg_starts, slots, out,         \
-                     out_stride, H, G, dim, vdim, q_scale, unit_eps)
-#define DELTA_PICK(T)                         \
-  do {                                        \
-    if (dim <= 32) DELTA_LAUNCH(T, 8);        \
-    else if (dim <= 64) DELTA_LAUNCH(T, 16);  \
-    else if (dim <= 128) DELTA_LAUNCH(T, 32); \
-    else DELTA_LAUNCH(T, 64);                 \
+  const int RPL = delta_rows_per_lane(dim);
+  float* prep = scratch;
+  float* beta = scratch + (long)n_tokens * H * 3 * DELTA_R * RPL;
+  const dim3 g1((unsigned)(((long)n_tokens * H + 3) / 4)), g2(n_segments, H, n_cb);
+#define DELTA_PREP(T)                                                                                                \
+  hipLaunchKernelGGL((gated_delta_prepare_kernel<T>), g1, dim3(256), 0, stream, (const T*)qkv, stride, q_at, k_at, a, \
+                     a_stride, dt_bias, a_log, b, b_stride, prep, beta, n_tokens, H, G, dim, RPL, q_scale, unit_eps)
+#define DELTA_RUN(T, R)                                                                                              \
+  hipLaunchKernelGGL((gated_delta_recurrence_kernel<T, R>), g2, dim3(LMSF_WAVE), 0, stream, (const T*)qkv, stride,    \
+                     v_at, prep, beta, state, state_stride, seg_starts, slots, out, out_stride, H, dim, vdim)
+#define DELTA_PICK(T)                  \
+  do {                                 \
+    DELTA_PREP(T);                     \
+    if (RPL == 1) DELTA_RUN(T, 1);     \
+    else if (RPL == 2) DELTA_RUN(T, 2);\
+    else if (RPL == 4) DELTA_RUN(T, 4);\
+    else if (RPL == 8) DELTA_RUN(T, 8);\
+    else DELTA_RUN(T, 16);             \
   } while (0)
   if (dtype == LMSF_F32) DELTA_PICK(float);
   else DELTA_PICK(bf16_t);
 #undef DELTA_PICK
-#undef DELTA_LAUNCH
+#undef DELTA_RUN
+#undef DELTA_PREP
   LMSF_LAUNCH_CHECK("gated_delta");
   return 0;
 }

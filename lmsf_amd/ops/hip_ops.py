@@ -968,7 +968,7 @@ class HipOps:
                     a_log: torch.Tensor, b: torch.Tensor, state: torch.Tensor, batch, heads: int, kv_heads: int,
                     dim: int, vdim: int, q_scale: float, unit_eps: float = 1e-6) -> torch.Tensor:
         """The gated delta rule over each request's tokens, the memory S [heads, dim, vdim] carried in ``state``
-        (float32 [slots, >= heads * dim * vdim]): S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, with
+        (float32 [slots, >= gated_delta_state_floats], laid out [heads, ceil(vdim / 4), dim, 4]): S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q, with
         q, k the unit vectors of columns q_at, k_at of ``qkv`` (kv_heads heads of dim; q times q_scale), v its columns
         from v_at (heads of vdim), beta = sigmoid(b [N, >= heads]) and g = exp(-exp(a_log [heads]) softplus(a + dt_bias))
         (``a`` float32 [N, heads * dim]). Returns the heads' o as float32 [N, heads * vdim]."""
@@ -988,10 +988,12 @@ class HipOps:
         self._state_view(state, self.gated_delta_state_floats(heads, dim, vdim), "gated_delta")
         _, seg_starts, slots, S = self._segments(batch, N)
         out = torch.empty((N, heads * vdim), dtype=torch.float32, device=qkv.device)
+        scratch = torch.empty(max(1, self.lib.lmsf_gated_delta_scratch_floats(N, int(heads), int(dim))),
+                              dtype=torch.float32, device=qkv.device)
         self._check(self.lib.lmsf_gated_delta(
             _ptr(qkv), _code(qkv.dtype), qkv.stride(0), int(q_at), int(k_at), int(v_at), _ptr(a), a.stride(0),
             _ptr(dt_bias), _ptr(a_log), _ptr(b), b.stride(0), _ptr(state), state.stride(0), _ptr(seg_starts), _ptr(slots),
-            _ptr(out), out.stride(0), N, S, int(heads), int(kv_heads), int(dim), int(vdim), float(q_scale),
+            _ptr(scratch), _ptr(out), out.stride(0), N, S, int(heads), int(kv_heads), int(dim), int(vdim), float(q_scale),
             float(unit_eps), self._stream()))
         return out
 
@@ -1507,6 +1509,18 @@ class HipOps:
             y = torch.empty((M, N), dtype=torch.float32, device=x.device)
             self._check(self.lib.lmsf_gemm_mid_reduce(_ptr(parts), _ptr(bias), _ptr(y), F32, y.stride(0), M, N, 2,
                                                       self._stream()))
+            return y
+        if (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and x.dim() == 2 and weight.dim() == 2
+                and M > self.mid_max_rows and weight.shape[1] == K and K < 128 and x.stride(1) == 1
+                and weight.stride(1) == 1 and (bias is None or (bias.shape == (N,) and bias.dtype == weight.dtype
+                                                                and bias.is_contiguous()))):
+            # a product over few columns (the second half of a low-rank pair): one launch of the plain kernel instead
+            # of pieces of ``mid_max_rows`` rows
+            self._dev(x, weight, bias)
+            y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+            self._check(self.lib.lmsf_gemm_plain(_ptr(x), _code(x.dtype), x.stride(0), _ptr(weight), _code(weight.dtype),
+                                                 weight.stride(0), _ptr(bias), _ptr(y), F32, y.stride(0), M, N, K,
+                                                 self._stream()))
             return y
         return self.linear(x, weight, bias, out_dtype=torch.float32)
 

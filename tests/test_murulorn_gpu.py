@@ -58,6 +58,14 @@ def batch_of(lens, slots, first_pos=None, ids=None, dev="cuda"):
                            host_seg_lens=list(lens), all_single=all(n == 1 for n in lens), replayed=False, aux={})
 
 
+def memory_as_the_kernel_keeps_it(S):
+    """[H, d, dv] -> the kernel's [H, ceil(dv / 4), d, 4], flat."""
+    H, d, dv = S.shape
+    pad = -dv % 4
+    S = torch.nn.functional.pad(S, (0, pad))
+    return S.reshape(H, d, (dv + pad) // 4, 4).permute(0, 2, 1, 3).reshape(-1)
+
+
 def table_of(dims, base, n=400):
     i = torch.arange(dims // 2, dtype=torch.float64)
     ang = torch.arange(n, dtype=torch.float64)[:, None] * (float(base) ** (-2.0 * i / dims))[None, :]
@@ -84,8 +92,13 @@ def test_the_delta_rule_against_the_recurrence(dtype, H, G, d, dv, lens):
     a = torch.randn((N, H * d + 3), generator=g)
     b = torch.randn((N, H + 2), generator=g) * 2
     dt_bias, a_log = torch.randn((H * d,), generator=g), torch.rand((H,), generator=g) * 2 - 1.5
-    state0 = torch.randn((5, H * d * dv + 3), generator=g) * 0.3
-    state0[0] = 0
+    mem = [torch.randn((H, d, dv), generator=g) * 0.3 for _ in range(5)]
+    mem[0] = torch.zeros((H, d, dv))
+    floats = o.gated_delta_state_floats(H, d, dv)
+    assert floats == H * ((dv + 3) // 4) * d * 4
+    state0 = torch.randn((5, floats + 3), generator=g)
+    for i in range(5):
+        state0[i, :floats] = memory_as_the_kernel_keeps_it(mem[i])
     pd = p.double()
     rep = H // G
     q = pd[:, 3:3 + G * d].reshape(N, G, d)
@@ -97,16 +110,16 @@ def test_the_delta_rule_against_the_recurrence(dtype, H, G, d, dv, lens):
     decay = torch.exp(-torch.exp(a_log.double())[None, :, None] * torch.nn.functional.softplus(
         a[:, :H * d].double() + dt_bias.double()).reshape(N, H, d))
     want = torch.empty((N, H * dv), dtype=torch.float64)
-    st = state0.double().clone()
+    st = [m.double() for m in mem]
     at = 0
     for n, slot in zip(lens, slots):
-        S = st[slot, :H * d * dv].reshape(H, d, dv).clone()
+        S = st[slot].clone()
         for t in range(at, at + n):
             S = S * decay[t][:, :, None]
             u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, k[t]))
             S = S + k[t][:, :, None] * u[:, None, :]
             want[t] = torch.einsum("hdv,hd->hv", S, q[t]).reshape(-1)
-        st[slot, :H * d * dv] = S.reshape(-1)
+        st[slot] = S
         at += n
     # the recurrence itself, from one segment and a zero state, is the plain implementation's function
     one = P.delta_rule(q[:lens[0]], k[:lens[0]], v[:lens[0]], beta[:lens[0]], decay[:lens[0]])
@@ -117,8 +130,10 @@ def test_the_delta_rule_against_the_recurrence(dtype, H, G, d, dv, lens):
                         batch_of(lens, slots), H, G, d, dv, d ** -0.5, 1e-6)
     assert got.dtype == torch.float32
     assert float((got.double().cpu() - want).abs().max()) <= 3e-5 * max(1.0, float(want.abs().max()))
-    assert float((state.cpu().double() - st).abs().max()) <= 3e-5 * max(1.0, float(st.abs().max()))
-    assert torch.equal(state.cpu()[:, H * d * dv:], state0[:, H * d * dv:])        # what lies behind is not touched
+    for i in range(5):
+        want_i = memory_as_the_kernel_keeps_it(st[i])
+        assert float((state.cpu()[i, :floats].double() - want_i).abs().max()) <= 3e-5 * max(1.0, float(want_i.abs().max()))
+    assert torch.equal(state.cpu()[:, floats:], state0[:, floats:])        # what lies behind is not touched
     assert torch.equal(state.cpu()[1], state0[1]) and torch.equal(state.cpu()[4], state0[4])
 
 
