@@ -988,7 +988,7 @@ class HipOps:
         self._state_view(state, self.gated_delta_state_floats(heads, dim, vdim), "gated_delta")
         _, seg_starts, slots, S = self._segments(batch, N)
         out = torch.empty((N, heads * vdim), dtype=torch.float32, device=qkv.device)
-        scratch = torch.empty(max(1, self.lib.lmsf_gated_delta_scratch_floats(N, int(heads), int(dim))),
+        scratch = torch.empty(max(1, self.lib.lmsf_gated_delta_scratch_floats(N, int(heads), int(dim), int(vdim))),
                               dtype=torch.float32, device=qkv.device)
         self._check(self.lib.lmsf_gated_delta(
             _ptr(qkv), _code(qkv.dtype), qkv.stride(0), int(q_at), int(k_at), int(v_at), _ptr(a), a.stride(0),
