@@ -986,14 +986,14 @@ class HipOps:
         if heads % kv_heads or dim > 256:
             raise ValueError("gated_delta: %d heads over %d key heads, keys of %d entries (at most 256)" % (heads, kv_heads, dim))
         self._state_view(state, self.gated_delta_state_floats(heads, dim, vdim), "gated_delta")
-        _, seg_starts, slots, S = self._segments(batch, N)
+        seg_of, seg_starts, slots, S = self._segments(batch, N)
         out = torch.empty((N, heads * vdim), dtype=torch.float32, device=qkv.device)
-        scratch = torch.empty(max(1, self.lib.lmsf_gated_delta_scratch_floats(N, int(heads), int(dim), int(vdim))),
+        scratch = torch.empty(max(1, self.lib.lmsf_gated_delta_scratch_floats(N, S, int(heads), int(dim), int(vdim))),
                               dtype=torch.float32, device=qkv.device)
         self._check(self.lib.lmsf_gated_delta(
             _ptr(qkv), _code(qkv.dtype), qkv.stride(0), int(q_at), int(k_at), int(v_at), _ptr(a), a.stride(0),
-            _ptr(dt_bias), _ptr(a_log), _ptr(b), b.stride(0), _ptr(state), state.stride(0), _ptr(seg_starts), _ptr(slots),
-            _ptr(scratch), _ptr(out), out.stride(0), N, S, int(heads), int(kv_heads), int(dim), int(vdim), float(q_scale),
+            _ptr(dt_bias), _ptr(a_log), _ptr(b), b.stride(0), _ptr(state), state.stride(0), _ptr(seg_of), _ptr(seg_starts),
+            _ptr(slots), _ptr(scratch), _ptr(out), out.stride(0), N, S, int(heads), int(kv_heads), int(dim), int(vdim), float(q_scale),
             float(unit_eps), self._stream()))
         return out
 

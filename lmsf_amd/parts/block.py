@@ -258,12 +258,18 @@ class TokenSideInput(Part):
     def tensors(self):
         return [t for t in (self.norm_weight,) if t is not None]
 
-    def forward(self, residual: torch.Tensor, ctx) -> None:
+    def forward(self, residual: torch.Tensor, ctx, x: Optional[torch.Tensor] = None, then=None) -> Optional[torch.Tensor]:
+        """``x``: the stream in the run's type, where the caller has it already. ``then``: a norm of the new stream
+        that the closing kernel computes as well; its result is returned."""
         ops = self.rt.ops
-        x = ops.group_norm(residual=residual, out_dtype=self.rt.dtype)          # the stream in the run's type
+        if x is None:
+            x = ops.group_norm(residual=residual, out_dtype=self.rt.dtype)      # the stream in the run's type
         g = ops.gate_table(self.gate.forward(x), ctx.token_ids, self.table, self.at)
         y = ops.linear_wide(g, self.proj.weight, None)
-        ops.group_norm(x=y, x_weight=self.norm_weight, residual=residual, x_eps=self.eps, want_out=False)
+        return ops.group_norm(x=y, x_weight=self.norm_weight, residual=residual, x_eps=self.eps,
+                              out_weight=then.weight if then is not None else None,
+                              out_eps=then.eps if then is not None else self.eps, out_dtype=self.rt.dtype,
+                              want_out=then is not None)
 
 
 @register_part("block", "sandwich")
@@ -276,7 +282,9 @@ class SandwichBlock(Block):
     embedding's output before the block (``inject``: the name of the matrix; a block that begins a pass of a loop over
     layers) and a per-layer input from the token added after it (``side``: the parameters of ``TokenSideInput``). The
     stream is float32; nothing is left to add when the block returns. The addition after the mixer and the norm
-    before the feed-forward are one kernel. The reference's only arrangement is the pre-norm one
+    before the feed-forward are one kernel; the addition after the feed-forward also hands the side input the stream in
+    the run's type; and the block's last kernel also computes the first norm of the block that always follows, where
+    that block does not replace the stream first (``link_next``). The reference's only arrangement is the pre-norm one
     (core/src/model_executor/models/llama/llama.rs:286-340)."""
 
     graph_safe = True
@@ -294,23 +302,46 @@ class SandwichBlock(Block):
         self.side = TokenSideInput("%s.%s" % (prefix, dict(side).pop("prefix", "side")), rt, hidden_size=hidden_size,
                                    **{k: v for k, v in dict(side).items() if k != "prefix"}) if side else None
         self._ffn_takes_ids = bool(getattr(feed_forward, "needs_token_ids", False))
+        self.next_norm = None       # the norm that the block after this one begins with, where the model has linked it
+
+    def link_next(self, following: Block) -> None:
+        """The model tells a block which block always runs after it: this one's last kernel then also computes that
+        one's first norm and leaves it in ``ctx.aux["prenormed"]``. Not where the following block replaces the stream
+        before its norm."""
+        if isinstance(following, SandwichBlock) and following.inject is None:
+            self.next_norm = following.norms["pre_mixer"]
 
     def children(self):
         return super().children() + [p for p in (self.inject, self.side) if p is not None]
+
+    def _close(self, norm, branch: torch.Tensor, residual: torch.Tensor, ctx) -> None:
+        """stream += norm(branch), then the side input; the last of these kernels also computes the next block's norm."""
+        ops = self.rt.ops
+        if self.side is None:
+            ahead = norm.add_normed(branch, residual, then=self.next_norm)
+        else:
+            # (no weight behind the sum: the kernel hands back the new stream itself, in the run's type)
+            x = ops.group_norm(x=branch, x_weight=norm.weight, residual=residual, groups=norm.groups, x_eps=norm.eps,
+                               out_dtype=self.rt.dtype)
+            ahead = self.side.forward(residual, ctx, x=x, then=self.next_norm)
+        if ahead is not None:
+            ctx.aux["prenormed"] = ahead
 
     def forward(self, branch: Optional[torch.Tensor], residual: torch.Tensor, ctx, binding: CacheBinding):
         if branch is not None:
             raise ValueError("sandwich takes no branch that is still to be added")
         n = self.norms
+        h = ctx.aux.pop("prenormed", None)
         if self.inject is not None:
             self.inject.forward(residual, ctx)
-        a = self.mixer.forward(n["pre_mixer"].forward(residual), ctx, binding)
+            h = None
+        if h is None:
+            h = n["pre_mixer"].forward(residual)
+        a = self.mixer.forward(h, ctx, binding)
         if self.has_ffn:
             h = n["post_mixer"].add_normed(a, residual, then=n["pre_ffn"])
             f = self.feed_forward.forward(h, token_ids=ctx.token_ids) if self._ffn_takes_ids else self.feed_forward.forward(h)
-            n["post_ffn"].add_normed(f, residual)
+            self._close(n["post_ffn"], f, residual, ctx)
         else:
-            n["post_mixer"].add_normed(a, residual)
-        if self.side is not None:
-            self.side.forward(residual, ctx)
+            self._close(n["post_mixer"], a, residual, ctx)
         return None

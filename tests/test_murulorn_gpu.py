@@ -30,13 +30,15 @@ def close(got, ref, dtype, scale=1.0):
     assert err <= tol * max(scale, float(ref.double().abs().max())), (err, float(ref.double().abs().max()))
 
 
-def check(got, ref, dtype, what, model_):
+def check(got, ref, dtype, what, model_, yardstick=0.0):
     """float32: three times what float32 rounding costs the plain implementation itself, where that is more than
-    TOL_F32; bfloat16: per position three times what rounding costs the plain implementation when it rounds what an
-    engine may keep in 16 bits."""
+    TOL_F32 (``yardstick``: that cost as the caller has measured it on other requests of the same model; one request
+    is one draw of the rounding errors, and how much a model amplifies them is the model's property); bfloat16: per
+    position three times what rounding costs the plain implementation when it rounds what an engine may keep in 16
+    bits."""
     cfg, w, toks = model_
     if dtype == "float32":
-        tol = max(TOL_F32, 3 * rel_err(plain_logits(cfg, w, toks, dtype=torch.float32), ref))
+        tol = max(TOL_F32, 3 * max(yardstick, rel_err(plain_logits(cfg, w, toks, dtype=torch.float32), ref)))
         assert rel_err(got, ref) < tol, (what, rel_err(got, ref), tol)
     else:
         ok, worst = within(got, ref, bfloat16_limits(cfg, w, toks, ref))
@@ -463,6 +465,9 @@ def test_a_configuration_drawn_at_random(tmp_path, seed, dtype):
     folder, cfg, w = make_model(tmp_path, cfg, seed, decisive=dtype == "bfloat16")
     reqs = {"r%d" % i: random_tokens(n, cfg["vocab"], 50 + i) for i, n in enumerate(lens)}
     refs = {rid: plain_logits(cfg, w, toks) for rid, toks in reqs.items()}
+    worst32 = 0.0
+    if dtype == "float32":
+        worst32 = max(rel_err(plain_logits(cfg, w, toks, dtype=torch.float32), refs[rid]) for rid, toks in reqs.items())
     alone = -(-max(lens) // page) + 1
     for what, steps, pages in (("whole", trace_whole(reqs), alone),
                                ("bulk then single", trace_bulk_then_single(reqs, tail=8), alone),
@@ -473,7 +478,7 @@ def test_a_configuration_drawn_at_random(tmp_path, seed, dtype):
         got = replay_in_process(core.executor, steps)
         for rid in reqs:
             assert torch.isfinite(got[rid]).all(), (what, rid, cfg)
-            check(got[rid], refs[rid], dtype, (what, rid, cfg, page), (cfg, w, reqs[rid]))
+            check(got[rid], refs[rid], dtype, (what, rid, cfg, page), (cfg, w, reqs[rid]), yardstick=worst32)
         core.storage.manager.check_invariants()
         assert core.storage.manager.num_free_state_slots() == 4
         del core
