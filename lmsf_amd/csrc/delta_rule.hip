@@ -21,12 +21,12 @@
 //
 // Two kernels. The first makes everything of a chunk ready that does not depend on S, side by side for all chunks: unit
 // vectors, decays, the vectors above in the order in which the second kernel's lanes read them, beta, A and B; and the
-// values as float32 in blocks of 16 columns. A chunk is four tokens of one request counted from the first token of its
+// values as float32 in blocks of 8 columns. A chunk is four tokens of one request counted from the first token of its
 // step's portion (the last chunk of a portion may hold fewer: the missing tokens have beta = 0 and k = q = 0). The
 // second runs the recurrence with a column's rows spread over 16 lanes (RPL = rows a lane holds, in registers; the key
-// size is padded to 16 RPL), four columns a wave and four waves a workgroup; the sum over a row of 16 lanes is four
+// size is padded to 16 RPL), four columns a wave and two waves a workgroup; the sum over a row of 16 lanes is four
 // additions through the vector unit's data-parallel path. What the steps read travels from global memory straight
-// into LDS a batch of chunks ahead (two buffers). Tokens of a request run one after the other; (request, head, 16
+// into LDS a batch of chunks ahead (two buffers). Tokens of a request run one after the other; (request, head, 8
 // columns) side by side. Measured at 2,048 tokens, 16 heads of 64 x 128: token by token with the operands asked for
 // four tokens ahead into registers 1,360 us (a step waited for memory), through LDS a batch ahead 767 us, with the
 // sums through the data-parallel path instead of the lane-permute instruction 376 us, four tokens at a time: see the
@@ -41,7 +41,7 @@
 
 #define DELTA_R 16            // lanes that share a column
 #define DELTA_CPW 4           // columns a wave holds
-#define DELTA_WAVES 4         // waves a workgroup
+#define DELTA_WAVES 2         // waves a workgroup (they share the operands in LDS, and LDS's rate is what a step waits for: see below)
 #define DELTA_COLS (DELTA_CPW * DELTA_WAVES)
 #define DELTA_CHUNK 4         // tokens a chunk
 
@@ -57,7 +57,29 @@ __host__ __device__ constexpr int delta_block_floats(int rpl) { return 13 * DELT
 // rows: rows of different segments never meet, and a segment's rows lie one behind the other.
 __device__ __forceinline__ long delta_chunk_row(int t0, int s, int t) { return t0 / DELTA_CHUNK + s + (t - t0) / DELTA_CHUNK; }
 
-// prep [H, chunk_rows, block] float32; vals [H, ceil(vdim / 16), val_rows, 16]: the values. A wave a (token, head);
+// The sum over a row of 16 lanes, in every lane of the row: four additions whose second operand comes through the
+// data-parallel path of the vector unit (neighbours within a quad, then the mirror image within 8 and within 16 lanes,
+// which by then hold equal sums on either side).
+template <int CTRL>
+__device__ __forceinline__ float delta_dpp(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float delta_sum16(float v) {
+  v += delta_dpp<0xB1>(v);      // quad_perm [1, 0, 3, 2]
+  v += delta_dpp<0x4E>(v);      // quad_perm [2, 3, 0, 1]
+  v += delta_dpp<0x141>(v);     // row_half_mirror
+  v += delta_dpp<0x140>(v);     // row_mirror
+  return v;
+}
+
+// The sum over the wave's 64 lanes, in every lane: the rows' sums, then the four rows' through scalar registers.
+__device__ __forceinline__ float delta_sum64(float v) {
+  v = delta_sum16(v);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0)) + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16)) +
+         __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32)) + __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+}
+
+// prep [H, chunk_rows, block] float32; vals [H, ceil(vdim / 8), val_rows, 8]: the values. A wave a (token, head);
 // the wave of a chunk's first token makes the chunk.
 template <typename T>
 __global__ __launch_bounds__(256) void gated_delta_prepare_kernel(
@@ -91,8 +113,8 @@ __global__ __launch_bounds__(256) void gated_delta_prepare_kernel(
         ssk += y * y;
       }
     }
-    iq[m] = q_scale / sqrtf(wave_sum(ssq) + unit_eps);
-    ik[m] = 1.f / sqrtf(wave_sum(ssk) + unit_eps);
+    iq[m] = q_scale / sqrtf(delta_sum64(ssq) + unit_eps);
+    ik[m] = 1.f / sqrtf(delta_sum64(ssk) + unit_eps);
   }
   const float rate = expf(a_log[h]);
   float* out = prep + ((long)h * chunk_rows + delta_chunk_row(t0, s, t)) * block;
@@ -137,9 +159,9 @@ __global__ __launch_bounds__(256) void gated_delta_prepare_kernel(
       }
   }
 #pragma unroll
-  for (int j = 0; j < 6; ++j) A[j] = wave_sum(A[j]);
+  for (int j = 0; j < 6; ++j) A[j] = delta_sum64(A[j]);
 #pragma unroll
-  for (int j = 0; j < 10; ++j) B[j] = wave_sum(B[j]);
+  for (int j = 0; j < 10; ++j) B[j] = delta_sum64(B[j]);
   if (lane == 0) {
     float* sc = out + 13 * DP;
 #pragma unroll
@@ -177,21 +199,6 @@ __device__ __forceinline__ void delta_load_vec(float* dst, const float* src) {
   }
 }
 
-// The sum over a row of 16 lanes, in every lane of the row: four additions whose second operand comes through the
-// data-parallel path of the vector unit (neighbours within a quad, then the mirror image within 8 and within 16 lanes,
-// which by then hold equal sums on either side).
-template <int CTRL>
-__device__ __forceinline__ float delta_dpp(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
-}
-__device__ __forceinline__ float delta_sum16(float v) {
-  v += delta_dpp<0xB1>(v);      // quad_perm [1, 0, 3, 2]
-  v += delta_dpp<0x4E>(v);      // quad_perm [2, 3, 0, 1]
-  v += delta_dpp<0x141>(v);     // row_half_mirror
-  v += delta_dpp<0x140>(v);     // row_mirror
-  return v;
-}
-
 template <int RPL>
 __global__ __launch_bounds__(DELTA_WAVES * LMSF_WAVE) void gated_delta_recurrence_kernel(
     const float* __restrict__ prep, const float* __restrict__ vals, long chunk_rows, long val_rows,
@@ -200,7 +207,8 @@ __global__ __launch_bounds__(DELTA_WAVES * LMSF_WAVE) void gated_delta_recurrenc
   constexpr int DP = DELTA_R * RPL, BLOCK = delta_block_floats(RPL), HC = delta_batch_chunks(RPL), HT = HC * DELTA_CHUNK;
   constexpr int OPS_BYTES = (HC * BLOCK * 4 + 1023) / 1024 * 1024, VAL_BYTES = (HT * DELTA_COLS * 4 + 1023) / 1024 * 1024;
   constexpr int N_OPS = OPS_BYTES / 1024, N_VAL = VAL_BYTES / 1024;     // transfers of 1 KB a batch
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // two buffers of [chunks | values]
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // two buffers of [chunks | values], two of results
+  float* results = reinterpret_cast<float*>(lds + 2 * (OPS_BYTES + VAL_BYTES));          // [2][HT][DELTA_COLS]
   const int s = blockIdx.x, h = blockIdx.y, cb = blockIdx.z;
   const int tid = threadIdx.x, wave = tid / LMSF_WAVE, lane = tid % LMSF_WAVE, c = lane / DELTA_R, r = lane % DELTA_R;
   const int col = cb * DELTA_COLS + wave * DELTA_CPW + c;
@@ -232,12 +240,24 @@ __global__ __launch_bounds__(DELTA_WAVES * LMSF_WAVE) void gated_delta_recurrenc
                              __builtin_amdgcn_readfirstlane(base + OPS_BYTES + n * 1024));
   };
   const int n_tok = t1 - t0, n_batches = (n_tok + HT - 1) / HT;
+  // A batch's results wait in LDS and go to memory while the next batch is worked on: stored as they come, the wait
+  // for the next batch's operands would also wait for the stores just issued, a trip to memory every batch.
+  auto flush = [&](int batch) {
+    const float* from = results + (batch & 1) * HT * DELTA_COLS;
+    const int n = min(HT, n_tok - batch * HT) * DELTA_COLS;
+    for (int e = tid; e < n; e += DELTA_WAVES * LMSF_WAVE) {
+      const int column = cb * DELTA_COLS + e % DELTA_COLS;
+      if (column < vdim) out[((long)t0 + (long)batch * HT + e / DELTA_COLS) * out_stride + h * vdim + column] = from[e];
+    }
+  };
   transfer(0, 0);
   for (int bt = 0; bt < n_batches; ++bt) {
     const int buf = bt & 1;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();                   // this batch has landed; everybody is done with the buffer of the one before
     if (bt + 1 < n_batches) transfer(bt + 1, buf ^ 1);
+    if (bt > 0) flush(bt - 1);
+    float* res = results + buf * HT * DELTA_COLS;
     const float* ops_ = reinterpret_cast<const float*>(lds + buf * (OPS_BYTES + VAL_BYTES));
     const float* val_ = reinterpret_cast<const float*>(lds + buf * (OPS_BYTES + VAL_BYTES) + OPS_BYTES);
     const int left = n_tok - bt * HT;                              // tokens from this batch's first on
@@ -264,7 +284,8 @@ __global__ __launch_bounds__(DELTA_WAVES * LMSF_WAVE) void gated_delta_recurrenc
         rs[m] = delta_sum16(rs[m]);
         ps[m] = delta_sum16(ps[m]);
       }
-      const float* sc = blk + 13 * DP;                             // beta [4], A [6], B [10]
+      float sc[20];                                                // beta [4], A [6], B [10]
+      delta_load_vec<20>(sc, blk + 13 * DP);
       float u[DELTA_CHUNK], o[DELTA_CHUNK];
       int ia = 0, ib = 0;
 #pragma unroll
@@ -291,14 +312,13 @@ __global__ __launch_bounds__(DELTA_WAVES * LMSF_WAVE) void gated_delta_recurrenc
 #pragma unroll
         for (int ii = 0; ii < RPL; ++ii) st[ii] = fmaf(kl[ii], u[m], st[ii]);
       }
-      if (r == 0 && col_ok) {
-        const long tk = (long)t0 + (long)bt * HT + jc * DELTA_CHUNK;
-#pragma unroll
-        for (int x = 0; x < DELTA_CHUNK; ++x)
-          if (jc * DELTA_CHUNK + x < left) out[(tk + x) * out_stride + h * vdim + col] = o[x];
-      }
+      // every lane of a column holds the four results: lane r < 4 of the column stores token r's (one store a chunk)
+      const float mine = r == 0 ? o[0] : r == 1 ? o[1] : r == 2 ? o[2] : o[3];
+      if (r < DELTA_CHUNK) res[(jc * DELTA_CHUNK + r) * DELTA_COLS + wave * DELTA_CPW + c] = mine;
     }
   }
+  __syncthreads();
+  flush(n_batches - 1);
   if (wave_ok) {
 #pragma unroll
     for (int ii = 0; ii < RPL; ++ii) {
@@ -332,7 +352,8 @@ static int launch_delta_recurrence(dim3 grid, hipStream_t stream, const float* p
                                    long val_rows, float* state, long state_stride, const int* seg_starts,
                                    const int* slots, float* out, long out_stride, int H, int dim, int vdim) {
   constexpr int BLOCK = delta_block_floats(RPL), HC = delta_batch_chunks(RPL), HT = HC * DELTA_CHUNK;
-  constexpr size_t smem = 2 * ((size_t)(HC * BLOCK * 4 + 1023) / 1024 * 1024 + (size_t)(HT * DELTA_COLS * 4 + 1023) / 1024 * 1024);
+  constexpr size_t smem = 2 * ((size_t)(HC * BLOCK * 4 + 1023) / 1024 * 1024 + (size_t)(HT * DELTA_COLS * 4 + 1023) / 1024 * 1024) +
+                          2 * (size_t)HT * DELTA_COLS * 4;
   auto kernel = gated_delta_recurrence_kernel<RPL>;
   static bool configured = false;   // per instantiation
   if (!configured) {
