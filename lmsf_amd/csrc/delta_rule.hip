@@ -199,12 +199,15 @@ __device__ __forceinline__ void delta_load_vec(float* dst, const float* src) {
   }
 }
 
-template <int RPL>
+// HC: chunks a batch holds (and LDS has room for, twice): delta_batch_chunks(RPL) for portions of prompts; 1 for a step
+// whose segments hold no more than a chunk (single tokens), where a workgroup then takes a few KB of LDS instead of
+// 59 and many of them share a compute unit.
+template <int RPL, int HC>
 __global__ __launch_bounds__(DELTA_WAVES * LMSF_WAVE) void gated_delta_recurrence_kernel(
     const float* __restrict__ prep, const float* __restrict__ vals, long chunk_rows, long val_rows,
     float* __restrict__ state, long state_stride, const int* __restrict__ seg_starts, const int* __restrict__ slots,
     float* __restrict__ out, long out_stride, int H, int dim, int vdim) {
-  constexpr int DP = DELTA_R * RPL, BLOCK = delta_block_floats(RPL), HC = delta_batch_chunks(RPL), HT = HC * DELTA_CHUNK;
+  constexpr int DP = DELTA_R * RPL, BLOCK = delta_block_floats(RPL), HT = HC * DELTA_CHUNK;
   constexpr int OPS_BYTES = (HC * BLOCK * 4 + 1023) / 1024 * 1024, VAL_BYTES = (HT * DELTA_COLS * 4 + 1023) / 1024 * 1024;
   constexpr int N_OPS = OPS_BYTES / 1024, N_VAL = VAL_BYTES / 1024;     // transfers of 1 KB a batch
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];  // two buffers of [chunks | values], two of results
@@ -229,17 +232,20 @@ __global__ __launch_bounds__(DELTA_WAVES * LMSF_WAVE) void gated_delta_recurrenc
       prep + ((long)h * chunk_rows + delta_chunk_row(t0, s, t0)) * BLOCK);
   const unsigned char* g_val = reinterpret_cast<const unsigned char*>(vals + (((long)h * n_cb + cb) * val_rows + t0) * DELTA_COLS);
   const unsigned lds0 = delta_lds_address(lds);
+  const int n_tok = t1 - t0, n_batches = (n_tok + HT - 1) / HT;
   auto transfer = [&](int batch, int buf) {
+    // (only what the batch holds)
+    const int toks = min(HT, n_tok - batch * HT), chunks = (toks + DELTA_CHUNK - 1) / DELTA_CHUNK;
+    const int n_ops = min(N_OPS, (chunks * BLOCK * 4 + 1023) / 1024), n_val = min(N_VAL, (toks * DELTA_COLS * 4 + 1023) / 1024);
     const unsigned base = lds0 + buf * (OPS_BYTES + VAL_BYTES);
     const int first = __builtin_amdgcn_readfirstlane(wave);          // (the same in every lane: the LDS base is a scalar)
-    for (int n = first; n < N_OPS; n += DELTA_WAVES)
+    for (int n = first; n < n_ops; n += DELTA_WAVES)
       delta_global_to_lds_16(g_ops + (long)batch * HC * BLOCK * 4 + n * 1024 + lane * 16,
                              __builtin_amdgcn_readfirstlane(base + n * 1024));
-    for (int n = first; n < N_VAL; n += DELTA_WAVES)
+    for (int n = first; n < n_val; n += DELTA_WAVES)
       delta_global_to_lds_16(g_val + (long)batch * HT * DELTA_COLS * 4 + n * 1024 + lane * 16,
                              __builtin_amdgcn_readfirstlane(base + OPS_BYTES + n * 1024));
   };
-  const int n_tok = t1 - t0, n_batches = (n_tok + HT - 1) / HT;
   // A batch's results wait in LDS and go to memory while the next batch is worked on: stored as they come, the wait
   // for the next batch's operands would also wait for the stores just issued, a trip to memory every batch.
   auto flush = [&](int batch) {
@@ -347,14 +353,14 @@ extern "C" long lmsf_gated_delta_scratch_floats(int n_tokens, int n_segments, in
          (long)H * n_cb * delta_val_rows(n_tokens, rpl) * DELTA_COLS + 256;
 }
 
-template <int RPL>
+template <int RPL, int HC>
 static int launch_delta_recurrence(dim3 grid, hipStream_t stream, const float* prep, const float* vals, long chunk_rows,
                                    long val_rows, float* state, long state_stride, const int* seg_starts,
                                    const int* slots, float* out, long out_stride, int H, int dim, int vdim) {
-  constexpr int BLOCK = delta_block_floats(RPL), HC = delta_batch_chunks(RPL), HT = HC * DELTA_CHUNK;
+  constexpr int BLOCK = delta_block_floats(RPL), HT = HC * DELTA_CHUNK;
   constexpr size_t smem = 2 * ((size_t)(HC * BLOCK * 4 + 1023) / 1024 * 1024 + (size_t)(HT * DELTA_COLS * 4 + 1023) / 1024 * 1024) +
                           2 * (size_t)HT * DELTA_COLS * 4;
-  auto kernel = gated_delta_recurrence_kernel<RPL>;
+  auto kernel = gated_delta_recurrence_kernel<RPL, HC>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -373,14 +379,15 @@ static int launch_delta_recurrence(dim3 grid, hipStream_t stream, const float* p
 // qkv: the (convolved, activated) q [N, G dim], k [N, G dim], v [N, H vdim] as columns q_at, k_at, v_at of one buffer
 // of ``dtype`` with row stride ``stride``; a: float32 [N, H dim] before bias and softplus; dt_bias float32 [H dim];
 // a_log float32 [H]; b: float32 [N, >= H] before the sigmoid; state float32 [slots, >= lmsf_gated_delta_state_floats];
-// seg_of [N], seg_starts [S + 1], slots [S]: the step's segments; scratch: lmsf_gated_delta_scratch_floats floats,
+// seg_of [N], seg_starts [S + 1], slots [S]: the step's segments; longest: the most tokens a segment holds, if the caller
+// knows (0: not known); scratch: lmsf_gated_delta_scratch_floats floats,
 // 16-byte aligned; out: float32 [N, H vdim], the heads' read-outs as they are.
 extern "C" int lmsf_gated_delta(const void* qkv, int dtype, long stride, int q_at, int k_at, int v_at, const float* a,
                                 long a_stride, const float* dt_bias, const float* a_log, const float* b,
                                 long b_stride, float* state, long state_stride, const int* seg_of,
                                 const int* seg_starts, const int* slots, float* scratch, float* out, long out_stride,
-                                int n_tokens, int n_segments, int H, int G, int dim, int vdim, float q_scale,
-                                float unit_eps, hipStream_t stream) {
+                                int n_tokens, int n_segments, int longest, int H, int G, int dim, int vdim,
+                                float q_scale, float unit_eps, hipStream_t stream) {
   LMSF_CHECK(qkv && a && dt_bias && a_log && b && state && seg_of && seg_starts && slots && out && scratch,
              "gated_delta: null pointer");
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "gated_delta: unknown dtype code %d", dtype);
@@ -405,9 +412,13 @@ extern "C" int lmsf_gated_delta(const void* qkv, int dtype, long stride, int q_a
   if (dtype == LMSF_F32) DELTA_PREP(float);
   else DELTA_PREP(bf16_t);
 #undef DELTA_PREP
-#define DELTA_RUN(R)                                                                                                \
-  launch_delta_recurrence<R>(g2, stream, prep, vals, chunk_rows, val_rows, state, state_stride, seg_starts, slots, out, \
-                             out_stride, H, dim, vdim)
+#define DELTA_RUN(R)                                                                                                   \
+  (small ? launch_delta_recurrence<R, 1>(g2, stream, prep, vals, chunk_rows, val_rows, state, state_stride, seg_starts, \
+                                         slots, out, out_stride, H, dim, vdim)                                         \
+         : launch_delta_recurrence<R, delta_batch_chunks(R)>(g2, stream, prep, vals, chunk_rows, val_rows, state,      \
+                                                             state_stride, seg_starts, slots, out, out_stride, H, dim, \
+                                                             vdim))
+  const bool small = longest > 0 && longest <= DELTA_CHUNK;
   const int rc = RPL == 1 ? DELTA_RUN(1) : RPL == 2 ? DELTA_RUN(2) : RPL == 4 ? DELTA_RUN(4) : RPL == 8 ? DELTA_RUN(8)
                                                                                                        : DELTA_RUN(16);
 #undef DELTA_RUN

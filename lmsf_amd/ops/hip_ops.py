@@ -993,7 +993,8 @@ class HipOps:
         self._check(self.lib.lmsf_gated_delta(
             _ptr(qkv), _code(qkv.dtype), qkv.stride(0), int(q_at), int(k_at), int(v_at), _ptr(a), a.stride(0),
             _ptr(dt_bias), _ptr(a_log), _ptr(b), b.stride(0), _ptr(state), state.stride(0), _ptr(seg_of), _ptr(seg_starts),
-            _ptr(slots), _ptr(scratch), _ptr(out), out.stride(0), N, S, int(heads), int(kv_heads), int(dim), int(vdim), float(q_scale),
+            _ptr(slots), _ptr(scratch), _ptr(out), out.stride(0), N, S,
+            1 if (getattr(batch, "all_single", False) and S == N) else 0, int(heads), int(kv_heads), int(dim), int(vdim), float(q_scale),
             float(unit_eps), self._stream()))
         return out
 

@@ -10,7 +10,7 @@ from typing import Optional
 from ..csrc import build as _build
 from .dispatch import ProductShape, Route, Tunables
 
-ABI_VERSION = 33
+ABI_VERSION = 34
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -60,7 +60,7 @@ _SIGNATURES = {
     "lmsf_gated_delta_state_floats": (c_long, [c_int, c_int, c_int]),
     "lmsf_gated_delta_scratch_floats": (c_long, [c_int, c_int, c_int, c_int, c_int]),
     "lmsf_gated_delta": (c_int, [_P, c_int, c_long, c_int, c_int, c_int, _P, c_long, _P, _P, _P, c_long, _P, c_long, _P, _P,
-                                 _P, _P, _P, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, _P]),
+                                 _P, _P, _P, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, _P]),
     "lmsf_head_rms_gate": (c_int, [_P, c_long, _P, _P, c_long, c_int, _P, c_long, c_int, c_int, c_int, c_int, c_float, _P]),
     "lmsf_table_moe_act": (c_int, [_P, c_int, c_long, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, c_long, _P, _P, _P,
                                    c_int, _P, _P, c_long, c_int, c_int, c_int, _P, _P, _P]),
