@@ -6,7 +6,7 @@
 // projections' results: q and k are made unit vectors per head, x / sqrt(sum x^2 + unit_eps), q times q_scale;
 // beta = sigmoid(b); g = exp(-exp(A_log_h) softplus(a + dt_bias)), one factor per head and key channel, acting on the
 // rows of S. H value heads and G query/key heads (head h reads q/k head h / (H / G)). S lives in the request's state
-// slot, float32 [H, dim, vdim], and is read once and written once a step.
+// slot in float32 and is read once and written once a step.
 //
 // The columns of S are independent of one another: column j only ever needs k, q, g, beta and v_j. Token by token a
 // step is a chain of dependent operations (two sums over the rows of a column, one after the other), and what bounds
@@ -29,9 +29,11 @@
 // into LDS a batch of chunks ahead (two buffers). Tokens of a request run one after the other; (request, head, 8
 // columns) side by side. Measured at 2,048 tokens, 16 heads of 64 x 128: token by token with the operands asked for
 // four tokens ahead into registers 1,360 us (a step waited for memory), through LDS a batch ahead 767 us, with the
-// sums through the data-parallel path instead of the lane-permute instruction 376 us, four tokens at a time: see the
-// design document. The state lies as [H, ceil(vdim / 4), dim, 4], so that a wave's part of it is one piece of memory;
-// a step of single tokens is the same kernels, bound by the memory's bytes: S in and out.
+// sums through the data-parallel path instead of the lane-permute instruction 376 us, four tokens at a time with one
+// store a chunk 293 us: about 160 instructions a chunk and lane with 4 rows a lane, one wave a SIMD, which is what bounds
+// it now (sharing the operands among 2 or 4 waves changed nothing). The state lies as [H, ceil(vdim / 4), dim, 4], so
+// that a wave's part of it is one piece of memory; a step of single tokens is the same kernels with room for one chunk
+// in LDS, bound by the memory's bytes: S in and out.
 //
 // A third kernel divides every head's o by its root mean square, multiplies by a weight over vdim (shared by the
 // heads) and by sigmoid or silu of a gate, and rounds to the run's type.
@@ -41,7 +43,7 @@
 
 #define DELTA_R 16            // lanes that share a column
 #define DELTA_CPW 4           // columns a wave holds
-#define DELTA_WAVES 2         // waves a workgroup (they share the operands in LDS, and LDS's rate is what a step waits for: see below)
+#define DELTA_WAVES 2         // waves a workgroup (they share the operands in LDS)
 #define DELTA_COLS (DELTA_CPW * DELTA_WAVES)
 #define DELTA_CHUNK 4         // tokens a chunk
 

@@ -16,7 +16,10 @@
 // The same kernels serve experts that a router chooses: ``ids`` null makes row n of the table token n's own choice (a
 // table [n_tokens, top] that a kernel of the step has just written, lmsf_moe_route below); ``pair_scale`` gives every
 // (token, choice) a float32 factor on the expert's *input*, y_e(s h), which the gate and up products take as a factor on
-// their results before these are rounded (W (s h) = s (W h)); ``base_scale`` a float32 factor per token on ``base``.
+// their results before these are rounded (W (s h) = s (W h)); ``base_scale`` a float32 factor per token on ``base``;
+// ``out_scale`` a float32 factor per (token, choice) on what the expert returns. Experts may also be of one matrix in,
+// y_e(h) = Wd_e relu(Wu_e h)^2 with Wgu [E, F, W] (lmsf_table_moe_act). A second router (lmsf_moe_route_groups) takes
+// softmax scores and chooses within the best groups of neighbouring experts.
 #include "common.h"
 
 #include <math.h>
