@@ -30,8 +30,9 @@
 // columns) side by side. Measured at 2,048 tokens, 16 heads of 64 x 128: token by token with the operands asked for
 // four tokens ahead into registers 1,360 us (a step waited for memory), through LDS a batch ahead 767 us, with the
 // sums through the data-parallel path instead of the lane-permute instruction 376 us, four tokens at a time with one
-// store a chunk 293 us: about 160 instructions a chunk and lane with 4 rows a lane, one wave a SIMD, which is what bounds
-// it now (sharing the operands among 2 or 4 waves changed nothing). The state lies as [H, ceil(vdim / 4), dim, 4], so
+// store a chunk 293 us: 132 vector, 36 scalar and 23 LDS instructions a chunk and wave with 4 rows a lane (counters), one
+// wave a SIMD, issuing in 58 % of its cycles: its own chain of instructions is what bounds it now (sharing the operands
+// among 2 or 4 waves changed nothing). The state lies as [H, ceil(vdim / 4), dim, 4], so
 // that a wave's part of it is one piece of memory; a step of single tokens is the same kernels with room for one chunk
 // in LDS, bound by the memory's bytes: S in and out.
 //
@@ -64,7 +65,8 @@ __device__ __forceinline__ long delta_chunk_row(int t0, int s, int t) { return t
 // which by then hold equal sums on either side).
 template <int CTRL>
 __device__ __forceinline__ float delta_dpp(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+  // (every lane has a source lane under these controls; with bound_ctrl set the compiler folds the move into the addition)
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
 __device__ __forceinline__ float delta_sum16(float v) {
   v += delta_dpp<0xB1>(v);      // quad_perm [1, 0, 3, 2]
