@@ -2,18 +2,23 @@
 kind of layer alone and the whole model through the engine's step function in float32 and bfloat16 under the ways of
 cutting a request into steps, keys at a window's edges and far away made to decide the logits, pages and state slots
 used again, long decoding from graphs, configurations drawn at random, and generation through the entry point."""
+import os
 import random
+import subprocess
 from types import SimpleNamespace
 
 import pytest
 import torch
 
 import plain_murulorn as P
-from helpers import random_tokens, replay_in_process, trace_bulk_then_single, trace_mixed, trace_portions, trace_whole
+from helpers import (random_tokens, replay_in_process, replay_with_program, trace_bulk_then_single, trace_mixed,
+                     trace_portions, trace_whole)
 from murulorn_helpers import (attn, bfloat16_limits, delta, dense, greedy, make_model, make_weights, model, moe,
                               plain_logits, rel_err, replay, single_layer, within)
 
 pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 DTYPES = [torch.float32, torch.bfloat16]
 TOL_F32 = 3e-5
@@ -494,3 +499,28 @@ def test_greedy_generation_through_the_entry_point(tmp_path):
     outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True))
     for p, o in zip(prompts, outs):
         assert list(o.outputs[0].token_ids) == greedy(cfg, w, p, 6)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_trace_runner_as_a_program(tmp_path, dtype):
+    """bin/trace_run as a child process on a model folder: it picks the class by config.json, and a mixed schedule in a
+    pool of 256 tokens with four state slots gives the plain logits."""
+    folder, cfg, w = make_model(tmp_path, "A", 4, decisive=dtype == "bfloat16")
+    lens = [90, 1, 37, 120, 5, 64]
+    reqs = {"r%d" % i: random_tokens(n, cfg["vocab"], 70 + i) for i, n in enumerate(lens)}
+    steps = trace_mixed(reqs, 256, seed=5)
+    got = replay_with_program(os.path.join(ROOT, "bin", "trace_run"), folder, dtype, steps, str(tmp_path / "out"), 256,
+                              cfg["vocab"])
+    for rid, toks in reqs.items():
+        check(got[rid], plain_logits(cfg, w, toks), dtype, rid, (cfg, w, toks))
+
+
+def test_the_command_line_generates(tmp_path):
+    folder, cfg, w = make_model(tmp_path, "D", 3)
+    prompt = random_tokens(11, cfg["vocab"], 9)
+    proc = subprocess.run([os.path.join(ROOT, "bin", "lmsf_generate"), "--model", folder, "--dtype", "float32",
+                           "--gpu-memory-utilization", "0.5", "--block-size", "8", "--max-model-len", "64",
+                           "--prompt-ids", ",".join(map(str, prompt)), "--temperature", "0", "--max-tokens", "8",
+                           "--ignore-eos"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert [int(t) for t in proc.stdout.strip().splitlines()[0].split()] == greedy(cfg, w, prompt, 8)
