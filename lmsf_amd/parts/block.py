@@ -308,8 +308,14 @@ class SandwichBlock(Block):
         """The model tells a block which block always runs after it: this one's last kernel then also computes that
         one's first norm and leaves it in ``ctx.aux["prenormed"]``. Not where the following block replaces the stream
         before its norm."""
-        if isinstance(following, SandwichBlock) and following.inject is None:
-            self.next_norm = following.norms["pre_mixer"]
+        if not isinstance(following, SandwichBlock) or following.inject is not None:
+            return
+        nxt = following.norms["pre_mixer"]
+        # (one kernel takes one number of groups for both of its norms: the side input's norm has one group, a
+        # block without side input closes with its own last norm)
+        closing = 1 if self.side is not None else self.norms["post_ffn" if self.has_ffn else "post_mixer"].groups
+        if getattr(nxt, "groups", None) == closing:
+            self.next_norm = nxt
 
     def children(self):
         return super().children() + [p for p in (self.inject, self.side) if p is not None]
