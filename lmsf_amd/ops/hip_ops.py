@@ -1489,14 +1489,19 @@ class HipOps:
                                                  _code(out_dtype), y.stride(0), M, N, K, self._stream()))
         return y
 
-    def linear_wide(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def linear_wide(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """x weight^T + bias in float32, for results that enter a recurrence (a step size, a gate). With many
         bfloat16 rows the product runs in the many-rows matrix-core kernel with K in two parts, whose float32 partial
         sums the reduction kernel adds up with the bias (the BLAS library's plans of this package write bfloat16
         only, and ``linear`` would cut the rows into pieces of ``mid_max_rows``: 16 launches for 2,048 rows);
-        otherwise it is ``linear`` with float32 output."""
+        otherwise it is ``linear`` with float32 output. ``out``: a contiguous float32 [M, N] tensor that takes the
+        result (not an operand of the product)."""
         M, K = x.shape
         N = weight.shape[0]
+        if out is not None and (tuple(out.shape) != (M, N) or out.dtype != torch.float32 or not out.is_contiguous()
+                                or out.device != x.device):
+            raise ValueError("linear_wide: out must be a contiguous float32 [%d, %d] tensor on x's device" % (M, N))
         if (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and M > self.mid_max_rows and x.dim() == 2
                 and weight.dim() == 2 and weight.shape[1] == K and K % 64 == 0 and K >= 128 and N % 8 == 0
                 and x.stride(1) == 1 and weight.stride(1) == 1 and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0
@@ -1507,7 +1512,7 @@ class HipOps:
             parts = torch.empty((2, M, N), dtype=torch.float32, device=x.device)
             self._check(self.lib.lmsf_gemm_large(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), None, None, 0,
                                                  M, N, K, 0, plan, _ptr(parts), 0, self._stream()))
-            y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+            y = out if out is not None else torch.empty((M, N), dtype=torch.float32, device=x.device)
             self._check(self.lib.lmsf_gemm_mid_reduce(_ptr(parts), _ptr(bias), _ptr(y), F32, y.stride(0), M, N, 2,
                                                       self._stream()))
             return y
@@ -1518,11 +1523,13 @@ class HipOps:
             # a product over few columns (the second half of a low-rank pair): one launch of the plain kernel instead
             # of pieces of ``mid_max_rows`` rows
             self._dev(x, weight, bias)
-            y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+            y = out if out is not None else torch.empty((M, N), dtype=torch.float32, device=x.device)
             self._check(self.lib.lmsf_gemm_plain(_ptr(x), _code(x.dtype), x.stride(0), _ptr(weight), _code(weight.dtype),
                                                  weight.stride(0), _ptr(bias), _ptr(y), F32, y.stride(0), M, N, K,
                                                  self._stream()))
             return y
+        if out is not None:
+            return self.linear(x, weight, bias, out_dtype=torch.float32, out=out)
         return self.linear(x, weight, bias, out_dtype=torch.float32)
 
     def linear_gated(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,

@@ -221,7 +221,7 @@ class StreamInjection(Part):
             raise ValueError("%s: the embedding did not keep its output for this step" % self.prefix)
         ops = self.rt.ops
         both = ops.concat_rows(residual, x0, self.rt.dtype)
-        residual.copy_(ops.linear_wide(both, self.proj.weight, None))
+        ops.linear_wide(both, self.proj.weight, None, out=residual)       # (the operand is the copy just made)
 
 
 class TokenSideInput(Part):

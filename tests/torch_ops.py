@@ -578,8 +578,9 @@ class TorchOps:
         y = y.to(out_dtype or x.dtype)
         return y if out is None else out.copy_(y)
 
-    def linear_wide(self, x, weight, bias=None):
-        return self.linear(x, weight, bias, out_dtype=torch.float32)
+    def linear_wide(self, x, weight, bias=None, out=None):
+        y = self.linear(x, weight, bias, out_dtype=torch.float32)
+        return y if out is None else out.copy_(y)
 
     def materialize(self, y):
         return y
